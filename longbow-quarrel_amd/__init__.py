@@ -1,12 +1,13 @@
 """longbow-quarrel on MI355X: a small model library with its own generation.
 
-One architecture (the Llama 3 dense decoder), one GPU, from a model folder
+Two architectures (the Llama 3 dense decoder; Vafodra, a hybrid of windowed attention with a sink, Mamba-2
+and the gated delta rule), one GPU, from a model folder
 (config.json + model.safetensors) to generated tokens, on hand-written gfx950
 kernels.
 """
 from . import models  # noqa: F401  (registers the architectures)
 from .api import QuarrelEngine, SamplerConfig, new_engine
-from .config import ConfigError, LlamaConfig, ModelConfig
+from .config import ConfigError, LlamaConfig, ModelConfig, VafodraConfig
 from .engine import Engine, GenerationResult, SequenceTooLong, StepEntry, generate
 from .loading import load_engine, random_engine
 from .sampling import NonFiniteLogits, SamplingParams
@@ -14,6 +15,6 @@ from .registry import register_architecture, registered_architectures
 from .weights import WeightError, write_model_folder
 
 __all__ = [
-    "ConfigError", "LlamaConfig", "ModelConfig", "Engine", "StepEntry", "load_engine", "random_engine",
+    "ConfigError", "LlamaConfig", "VafodraConfig", "ModelConfig", "Engine", "StepEntry", "load_engine", "random_engine",
     "GenerationResult", "generate", "SamplingParams", "NonFiniteLogits", "SequenceTooLong", "QuarrelEngine", "SamplerConfig", "new_engine", "register_architecture", "registered_architectures", "WeightError", "write_model_folder",
 ]

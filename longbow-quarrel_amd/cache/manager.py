@@ -21,7 +21,7 @@ from typing import Dict, List, Mapping, Optional, Tuple
 
 import torch
 
-from ..parts.base import CacheNeed, KVNeed, LayerCache, StateNeed
+from ..parts.base import CacheNeed, KVNeed, LayerCache, MultiCache, StateNeed
 from .slots import BLOCK_SIZE, CacheFull, FreeList
 
 
@@ -85,7 +85,7 @@ class KVGroup(CacheGroup):
         self.max_slots = int(max_slots)
         self.blocks = FreeList(self.n_blocks, "cache block")
         shape_k = (len(layers), self.n_blocks, need.kv_heads, BLOCK_SIZE, need.head_dim)
-        shape_v = (len(layers), self.n_blocks, need.kv_heads, need.head_dim, BLOCK_SIZE)
+        shape_v = (len(layers), self.n_blocks, need.kv_heads, need.v_dim, BLOCK_SIZE)
         # reads are bounded by each sequence's length, but kernels load whole tiles of a block and
         # mask afterwards: what they load must at least be finite numbers
         self.k = torch.zeros(shape_k, dtype=dtype, device=device)
@@ -150,7 +150,8 @@ class KVGroup(CacheGroup):
             return
         first_needed = max(0, length - w + 1) // BLOCK_SIZE
         owned = self.owned[slot]
-        for b in range(min(first_needed, len(owned))):
+        kept = blocks_for(self.need.keep_first)  # the blocks of the first positions stay for good
+        for b in range(kept, min(first_needed, len(owned))):
             if owned[b] is not None:
                 self.blocks.give(owned[b])
                 owned[b] = None
@@ -175,6 +176,51 @@ class StateGroup(CacheGroup):
 
     def clear(self, slot: int) -> None:
         self.data[:, slot].zero_()
+
+
+class MultiGroup(CacheGroup):
+    """The groups of a `MultiNeed`, one for each of its needs, behind the interface of one group: what grows
+    is asked of every member (the member that lacks the most blocks, or has the fewest free, answers)."""
+
+    def __init__(self, members: List[CacheGroup]) -> None:
+        self.members = list(members)
+        self.layers = list(members[0].layers) if members else []
+
+    def layer_view(self, layer: int) -> MultiCache:
+        return MultiCache([g.layer_view(layer) for g in self.members])
+
+    def free_blocks(self) -> int:
+        return min((g.free_blocks() for g in self.members), default=1 << 60)
+
+    def taken_blocks(self) -> int:
+        return max((g.taken_blocks() for g in self.members), default=0)
+
+    def blocks_for(self, tokens: int) -> int:
+        return max((g.blocks_for(tokens) for g in self.members), default=0)
+
+    def blocks_missing(self, slot: int, new_len: int) -> int:
+        # members' pools have one size and are asked together: the largest lack is what must be free in each
+        return max((g.blocks_missing(slot, new_len) for g in self.members), default=0)
+
+    def ensure(self, slot: int, new_len: int) -> None:
+        for g in self.members:
+            g.ensure(slot, new_len)
+
+    def reserved(self) -> None:
+        for g in self.members:
+            g.reserved()
+
+    def trim(self, slot: int, length: int) -> None:
+        for g in self.members:
+            g.trim(slot, length)
+
+    def release(self, slot: int) -> None:
+        for g in self.members:
+            g.release(slot)
+
+    def clear(self, slot: int) -> None:
+        for g in self.members:
+            g.clear(slot)
 
 
 class CacheManager:
@@ -203,13 +249,24 @@ class CacheManager:
             for layer in layers:
                 self._owner[layer] = g
 
+    def _flat(self) -> List[CacheGroup]:
+        out: List[CacheGroup] = []
+        todo = list(self.groups)
+        while todo:
+            g = todo.pop(0)
+            if isinstance(g, MultiGroup):
+                todo = list(g.members) + todo
+            else:
+                out.append(g)
+        return out
+
     @property
     def kv_groups(self) -> List[KVGroup]:
-        return [g for g in self.groups if isinstance(g, KVGroup)]
+        return [g for g in self._flat() if isinstance(g, KVGroup)]
 
     @property
     def state_groups(self) -> List[StateGroup]:
-        return [g for g in self.groups if isinstance(g, StateGroup)]
+        return [g for g in self._flat() if isinstance(g, StateGroup)]
 
     # ---- slots ------------------------------------------------------------------------
     def acquire(self) -> int:

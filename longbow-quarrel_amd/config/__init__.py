@@ -1,5 +1,6 @@
 """Typed configurations read from a model folder's config.json."""
 from .base import ConfigError, ModelConfig, read_config_json
 from .llama import LlamaConfig, RopeScaling
+from .vafodra import VafodraConfig
 
-__all__ = ["ConfigError", "ModelConfig", "read_config_json", "LlamaConfig", "RopeScaling"]
+__all__ = ["ConfigError", "ModelConfig", "read_config_json", "LlamaConfig", "RopeScaling", "VafodraConfig"]

@@ -46,9 +46,12 @@ class ModelSpec:
     max_positions: Optional[int] = None  # the longest sequence the architecture's configuration allows
 
 
-def token_table(name: str, vocab_size: int, width: int) -> PartSpec:
-    """The plain embedding: x = E[token]."""
-    return PartSpec("token_table", {"name": name, "vocab_size": vocab_size, "width": width})
+def token_table(name: str, vocab_size: int, width: int, scale: float = 1.0) -> PartSpec:
+    """The plain embedding: x = E[token] (times `scale`, where a model has such a constant)."""
+    params = {"name": name, "vocab_size": vocab_size, "width": width}
+    if scale != 1.0:
+        params["scale"] = scale
+    return PartSpec("token_table", params)
 
 
 class DecoderModel:
@@ -166,7 +169,10 @@ class DecoderModel:
             else:
                 pending = block.forward(x, pending, ctx, cache)
             if ctx.observe is not None:
-                ctx.observe(f"run {i}", x, None if isinstance(pending, RowStats) else pending)
+                ctx.observe(f"run {i}", x, None if isinstance(pending, RowStats) or hasattr(pending, "settle")
+                            else pending)
+        if hasattr(pending, "settle"):  # a pending object of a block's own kind adds itself to the stream
+            pending = pending.settle(x, ctx)
         if n_want == 0:
             return None
         ctx.ws.next_run()

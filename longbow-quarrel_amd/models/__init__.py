@@ -1,2 +1,2 @@
 """Architectures.  Importing the package registers them."""
-from . import llama  # noqa: F401
+from . import llama, vafodra  # noqa: F401

@@ -106,12 +106,20 @@ class CacheNeed:
 
 @dataclass(frozen=True)
 class KVNeed(CacheNeed):
-    """Keys and values per position: `kv_heads` x `head_dim` each; window = 0 keeps all positions,
-    window = w keeps the last w (older blocks go back to the pool)."""
+    """Keys and values per position: `kv_heads` x `head_dim` each (values `value_dim` wide where that is
+    set and differs); window = 0 keeps all positions, window = w keeps the last w (older blocks go back to
+    the pool), except the blocks that hold the first `keep_first` positions, which every later query still
+    sees."""
 
     kv_heads: int
     head_dim: int
     window: int = 0
+    value_dim: int = 0  # 0: as wide as the keys
+    keep_first: int = 0
+
+    @property
+    def v_dim(self) -> int:
+        return self.value_dim or self.head_dim
 
     def make_group(self, runs, n_blocks, max_slots, dtype, device):
         from ..cache.manager import KVGroup
@@ -128,6 +136,19 @@ class StateNeed(CacheNeed):
     def make_group(self, runs, n_blocks, max_slots, dtype, device):
         from ..cache.manager import StateGroup
         return StateGroup(self, runs, max_slots, device)
+
+
+@dataclass(frozen=True)
+class MultiNeed(CacheNeed):
+    """Several needs of one mixer (keys and values beside a recurrent state, a state beside the last inputs
+    of a short convolution): every need gets its own group, and the mixer receives a `MultiCache` whose
+    `parts` are the groups' views in the order of `needs`."""
+
+    needs: Tuple[CacheNeed, ...]
+
+    def make_group(self, runs, n_blocks, max_slots, dtype, device):
+        from ..cache.manager import MultiGroup
+        return MultiGroup([n.make_group(runs, n_blocks, max_slots, dtype, device) for n in self.needs])
 
 
 # ---- build-time and step-time context ---------------------------------------------
@@ -297,6 +318,17 @@ class LayerCache:
         return replace(self, write=False)
 
 
+@dataclass
+class MultiCache:
+    """What a mixer with a `MultiNeed` sees: one view for each of its needs."""
+
+    parts: List[Any]
+    write: bool = True
+
+    def read_only(self) -> "MultiCache":
+        return MultiCache([p.read_only() for p in self.parts], write=False)
+
+
 # ---- the parts -----------------------------------------------------------------------
 
 
@@ -406,6 +438,8 @@ class Mixer(Part):
     # NormedRows instead of a tensor.  takes_residual_sink: forward has a keyword `sink`.
     takes_normed_rows = False
     takes_residual_sink = False
+    #: forward has a keyword `out`, a float32 [rows, width] buffer of the caller's that the result is written to
+    takes_out = False
 
     def cache_need(self):
         """KVNeed, StateNeed or None."""
@@ -439,6 +473,7 @@ class FeedForward(Part):
 
     takes_normed_rows = False    # as for Mixer
     takes_residual_sink = False
+    takes_out = False
 
     def forward(self, h: torch.Tensor, ctx: StepContext) -> torch.Tensor:
         raise NotImplementedError

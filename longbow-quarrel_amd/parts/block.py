@@ -45,6 +45,8 @@ class PreNormBlock(Block):
     @staticmethod
     def _normed(norm, x: torch.Tensor, pending, ctx: StepContext, consumer):
         """The rows for `consumer`: normalised now, or left for it to normalise where it can."""
+        if hasattr(pending, "settle"):  # a pending object of another block's own kind: it adds itself
+            pending = pending.settle(x, ctx)
         if isinstance(pending, RowStats):
             if consumer.takes_normed_rows and pending.norm is norm and pending.scaled is not None:
                 return NormedRows(x, norm, pending)
@@ -65,3 +67,82 @@ class PreNormBlock(Block):
             pending = self.ffn.forward(h, ctx, sink=sink)
             return sink.stats if pending is None else pending
         return self.ffn.forward(h, ctx)
+
+
+class ScaledDelta:
+    """What a `ParallelBlock` leaves pending: the stream is x + scale * (sum of `pieces` [n, rows, width]).
+    A consumer that cannot add it on its way calls `settle`, which brings x up to date."""
+
+    def __init__(self, pieces: torch.Tensor, scale: float) -> None:
+        self.pieces, self.scale = pieces, scale
+
+    def settle(self, x: torch.Tensor, ctx: StepContext) -> None:
+        ctx.kernels.add_scaled(x, self.pieces, self.scale)
+        return None
+
+
+@BLOCKS.register("parallel")
+class ParallelBlock(Block):
+    """One norm, whose output both sub-layers read: x += scale * (mixer(norm(x)) + ffn(norm(x))).  The
+    feed-forward may be absent (`feed_forward=None`).  The add rides on the next block's norm where that
+    norm takes a scaled delta (`takes_delta_scale`); otherwise the block adds before it returns."""
+
+    takes_next_norm = True
+
+    def __init__(self, mixer: PartSpec, norm: PartSpec, feed_forward: Optional[PartSpec] = None,
+                 scale: float = 1.0) -> None:
+        self.mixer = build_part(MIXERS, mixer)
+        self.ffn = build_part(FEED_FORWARDS, feed_forward) if feed_forward is not None else None
+        self.norm = build_part(NORMS, norm)
+        self.scale = float(scale)
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(p.graph_safe for p in self.parts())
+
+    @property
+    def first_norm(self):
+        return self.norm
+
+    def parts(self):
+        return tuple(p for p in (self.norm, self.mixer, self.ffn) if p is not None)
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [s for p in self.parts() for s in p.tensor_specs()]
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], env: BuildEnv) -> None:
+        super().bind(tensors, env)
+        for p in self.parts():
+            p.bind(tensors, env)
+
+    def forward(self, x: torch.Tensor, pending, ctx: StepContext, cache: Optional[LayerCache], next_norm=None):
+        kn = ctx.kernels
+        if isinstance(pending, ScaledDelta) and getattr(self.norm, "takes_delta_scale", False):
+            h = self.norm.forward(x, ctx, delta=pending.pieces, delta_scale=pending.scale)
+        else:
+            if hasattr(pending, "settle"):
+                pending = pending.settle(x, ctx)
+            h = self.norm.forward(x, ctx, delta=None if isinstance(pending, RowStats) else pending)
+        subs = [(self.mixer, (h, ctx, cache))] + ([(self.ffn, (h, ctx))] if self.ffn is not None else [])
+        pieces = ctx.ws.alloc((len(subs), x.shape[0], x.shape[1]), torch.float32)
+        for i, (part, args) in enumerate(subs):
+            if part.takes_out:
+                part.forward(*args, out=pieces[i])
+            else:  # a part that returns its result, whole or as pieces of its own
+                self._copy_into(kn, part.forward(*args), pieces[i])
+        # whoever looks at the stream between blocks (`ctx.observe`), and a norm that takes no scaled delta,
+        # gets the stream whole
+        if ctx.observe is None and next_norm is not None and getattr(next_norm, "takes_delta_scale", False):
+            return ScaledDelta(pieces, self.scale)
+        kn.add_scaled(x, pieces, self.scale)
+        return None
+
+    @staticmethod
+    def _copy_into(kn, got: torch.Tensor, out: torch.Tensor) -> None:
+        """A part's own result, whole [rows, width] or pieces [n, rows, width], summed into `out`."""
+        if got.dim() == 3:
+            kn.cast(got[0], out)
+            for piece in got[1:]:
+                kn.add(out, piece)
+        else:
+            kn.cast(got, out)

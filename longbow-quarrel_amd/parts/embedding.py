@@ -17,8 +17,9 @@ class TokenTable(Embedding):
     # form of it (`parts.base.product_weight`) in its place
     table_is_for_kernels = True
 
-    def __init__(self, name: str, vocab_size: int, width: int) -> None:
-        self.name, self.vocab_size, self.width = name, int(vocab_size), int(width)
+    def __init__(self, name: str, vocab_size: int, width: int, scale: float = 1.0) -> None:
+        """`scale`: x = scale * E[token] (a model's own constant; the product is taken in 32-bit)."""
+        self.name, self.vocab_size, self.width, self.scale = name, int(vocab_size), int(width), float(scale)
         self.table: Optional[torch.Tensor] = None
 
     def tensor_specs(self) -> List[TensorSpec]:
@@ -30,5 +31,8 @@ class TokenTable(Embedding):
 
     def forward(self, ctx: StepContext) -> torch.Tensor:
         x = ctx.ws.alloc((ctx.rows, self.width), torch.float32, keep=True)
-        ctx.kernels.embed(self.table, ctx.tokens, x)
+        if self.scale == 1.0:
+            ctx.kernels.embed(self.table, ctx.tokens, x)
+        else:
+            ctx.kernels.embed(self.table, ctx.tokens, x, scale=self.scale)
         return x

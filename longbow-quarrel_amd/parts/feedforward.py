@@ -67,3 +67,52 @@ class SwiGLU(FeedForward):
                 project(kn, ctx, h, self.w_gate_up, gu)
             kn.swiglu(gu, act)
         return project_into(kn, ctx, act, self.w_down, sink)
+
+
+@FEED_FORWARDS.register("glu")
+class GatedLinearUnit(FeedForward):
+    """down(act(gate(h)) * up(h)) with a choice of `activation` ("relu", "silu", "gelu_tanh"); no biases.  gate
+    and up are one matrix product whose 32-bit result the activation kernel reads."""
+
+    graph_safe = True
+    ACTIVATIONS = ("silu", "relu", "gelu_tanh")
+
+    def __init__(self, width: int, inner: int, prefix: str, activation: str = "silu",
+                 names: Optional[Mapping[str, str]] = None) -> None:
+        if activation not in self.ACTIVATIONS:
+            raise ValueError(f"unknown activation {activation!r}; known: {', '.join(self.ACTIVATIONS)}")
+        self.width, self.inner, self.activation = int(width), int(inner), activation
+        n = {"gate": "gate", "up": "up", "down": "down"}
+        n.update(names or {})
+        self.names: Dict[str, str] = {key: f"{prefix}.{val}" for key, val in n.items()}
+        self.w_gate_up: Optional[torch.Tensor] = None
+        self.w_down: Optional[torch.Tensor] = None
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [
+            TensorSpec(self.names["gate"], (self.inner, self.width)),
+            TensorSpec(self.names["up"], (self.inner, self.width)),
+            TensorSpec(self.names["down"], (self.width, self.inner)),
+        ]
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], env: BuildEnv) -> None:
+        super().bind(tensors, env)
+        gate, up = tensors[self.names["gate"]], tensors[self.names["up"]]
+        if gate.dtype != up.dtype:
+            raise ValueError(f"{self.names['gate']}: gate and up projections are stored in different dtypes")
+        self.w_gate_up = product_weight(env, torch.cat([gate, up], dim=0))
+        self.w_down = product_weight(env, tensors[self.names["down"]])
+
+    takes_out = True
+
+    def forward(self, h, ctx: StepContext, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        kn = ctx.kernels
+        rows = h.shape[0]
+        gu = ctx.ws.alloc((rows, 2 * self.inner), torch.float32)
+        project(kn, ctx, h, self.w_gate_up, gu)
+        act = ctx.ws.alloc((rows, self.inner), ctx.dtype)
+        kn.glu(gu, act, self.activation)
+        if out is None:
+            out = ctx.ws.alloc((rows, self.width), torch.float32)
+        project(kn, ctx, act, self.w_down, out)
+        return out

@@ -33,3 +33,40 @@ class RMSNorm(Norm):
         out = ctx.ws.alloc(x.shape, ctx.dtype)
         ctx.kernels.rmsnorm(x, self.weight, self.eps, out, delta=delta)
         return out
+
+
+@NORMS.register("dynamic_tanh")
+class DynamicTanh(Norm):
+    """y = tanh(alpha x) w + b with a learned scalar alpha: an element-wise squashing in a norm's place, which
+    computes no mean and no variance (Zhu, Chen, He, LeCun, Liu: "Transformers without Normalization").
+    The tanh is taken in 32-bit.  `names` gives the tensors of the weight, the bias and alpha."""
+
+    graph_safe = True
+    deferrable = False  # there are no row statistics that a product could fold in
+    takes_delta_scale = True  # forward(..., delta_scale=s) adds s * delta
+
+    def __init__(self, width: int, name: str, bias_name: Optional[str] = None, alpha_name: Optional[str] = None) -> None:
+        self.width = int(width)
+        self.name = name
+        self.bias_name = bias_name or name + ".b"
+        self.alpha_name = alpha_name or name + ".alpha"
+        self.weight: Optional[torch.Tensor] = None
+        self.bias: Optional[torch.Tensor] = None
+        self.alpha: Optional[torch.Tensor] = None
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [TensorSpec(self.name, (self.width,), kind=VECTOR32, init="around_one"),
+                TensorSpec(self.bias_name, (self.width,), kind=VECTOR32, init="normal"),
+                TensorSpec(self.alpha_name, (), kind=VECTOR32, init="around_one")]
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], env: BuildEnv) -> None:
+        super().bind(tensors, env)
+        self.weight = tensors[self.name].contiguous()
+        self.bias = tensors[self.bias_name].contiguous()
+        self.alpha = tensors[self.alpha_name].reshape(1).contiguous()  # read on the device: no copy to the host
+
+    def forward(self, x: torch.Tensor, ctx: StepContext, delta: Optional[torch.Tensor] = None,
+                delta_scale: float = 1.0) -> torch.Tensor:
+        out = ctx.ws.alloc(x.shape, ctx.dtype)
+        ctx.kernels.dynamic_tanh(x, self.weight, self.bias, self.alpha, out, delta=delta, delta_scale=delta_scale)
+        return out

@@ -1,0 +1,108 @@
+"""Attention over a sliding window that also keeps the first tokens of the sequence, with a sink.
+
+q = h Wq^T, k = h Wk^T, v = h Wv^T without biases; keys are `key_dim` wide, values `value_dim` (they may
+differ); query head h reads kv head h // (heads / kv_heads).  Position i sees position j when j <= i and
+(i - j < window or j < keep_first); window = 0 means every earlier position.  With `sink` the softmax has one
+more term in its denominator, a key of score 0 that carries no value: p_j = e^(s_j) / (1 + sum e^(s_j)), so a
+query may look at nothing (Xiao, Tian, Chen, Han, Lewis: "Efficient Streaming Language Models with Attention
+Sinks" keeps first tokens for the same purpose).  With `head_gate` every head's result is multiplied by the
+sigmoid of one more projection of h, a number per head.  Scores, probabilities and the sums over values are
+32-bit whatever the run's dtype.  A position encoding is optional (`position=None`: positions do not enter
+the scores).
+
+All projections of h are one matrix product ([q | k | v | gate]).
+"""
+from __future__ import annotations
+
+from typing import Dict, List, Mapping, Optional
+
+import torch
+
+from .base import (MIXERS, POSITION_ENCODINGS, BuildEnv, KVNeed, LayerCache, Mixer, PartSpec, StepContext,
+                   TensorSpec, build_part, product_weight, project)
+
+
+@MIXERS.register("sink_window_attention")
+class SinkWindowAttention(Mixer):
+    takes_out = True
+
+    def __init__(self, width: int, heads: int, kv_heads: int, key_dim: int, value_dim: int, scale: float,
+                 prefix: str, window: int = 0, keep_first: int = 0, sink: bool = True, head_gate: bool = False,
+                 position: Optional[PartSpec] = None, names: Optional[Mapping[str, str]] = None) -> None:
+        if heads % kv_heads != 0:
+            raise ValueError(f"{heads} heads cannot share {kv_heads} kv heads evenly")
+        if window < 0 or keep_first < 0:
+            raise ValueError("window and keep_first must not be negative")
+        self.width, self.heads, self.kv_heads = int(width), int(heads), int(kv_heads)
+        self.key_dim, self.value_dim = int(key_dim), int(value_dim)
+        self.scale, self.window, self.keep_first = float(scale), int(window), int(keep_first)
+        self.sink, self.head_gate = bool(sink), bool(head_gate)
+        n = {"q": "q", "k": "k", "v": "v", "gate": "g", "o": "o"}
+        n.update(names or {})
+        self.names: Dict[str, str] = {key: f"{prefix}.{val}" for key, val in n.items()}
+        self.position = build_part(POSITION_ENCODINGS, position) if position is not None else None
+        self.q_width = self.heads * self.key_dim
+        self.k_width = self.kv_heads * self.key_dim
+        self.v_width = self.kv_heads * self.value_dim
+        self.o_width = self.heads * self.value_dim
+        self.w_in: Optional[torch.Tensor] = None
+        self.w_o: Optional[torch.Tensor] = None
+
+    @property
+    def graph_safe(self) -> bool:
+        return self.position is None or self.position.graph_safe
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        specs = [
+            TensorSpec(self.names["q"], (self.q_width, self.width)),
+            TensorSpec(self.names["k"], (self.k_width, self.width)),
+            TensorSpec(self.names["v"], (self.v_width, self.width)),
+        ]
+        if self.head_gate:
+            specs.append(TensorSpec(self.names["gate"], (self.heads, self.width)))
+        specs.append(TensorSpec(self.names["o"], (self.width, self.o_width)))
+        return specs + (self.position.tensor_specs() if self.position is not None else [])
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], env: BuildEnv) -> None:
+        super().bind(tensors, env)
+        mats = [tensors[self.names[key]] for key in ("q", "k", "v") + (("gate",) if self.head_gate else ())]
+        if len({m.dtype for m in mats}) != 1:
+            raise ValueError(f"{self.names['q']}: the projections of one input are stored in different dtypes")
+        self.w_in = product_weight(env, torch.cat(mats, dim=0))
+        self.w_o = product_weight(env, tensors[self.names["o"]])
+        if self.position is not None:
+            self.position.bind(tensors, env)
+
+    def cache_need(self) -> KVNeed:
+        # a window that keeps first tokens still gives its middle blocks back
+        return KVNeed(self.kv_heads, self.key_dim, self.window, self.value_dim, self.keep_first if self.window else 0)
+
+    def forward(self, h: torch.Tensor, ctx: StepContext, cache: Optional[LayerCache],
+                out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        if cache is None or cache.k is None:
+            raise RuntimeError("attention needs a key/value cache")
+        kn = ctx.kernels
+        rows = h.shape[0]
+        total = self.q_width + self.k_width + self.v_width + (self.heads if self.head_gate else 0)
+        total_padded = (total + 3) // 4 * 4  # rows of the product start on 16 bytes
+        # q, k and v in the run's dtype (what the cache holds); the gate's logits ride in the same product
+        proj = ctx.ws.alloc((rows, total_padded), ctx.dtype)[:, :total]
+        project(kn, ctx, h, self.w_in, proj)
+        q = proj[:, : self.q_width]
+        k = proj[:, self.q_width : self.q_width + self.k_width]
+        v = proj[:, self.q_width + self.k_width : self.q_width + self.k_width + self.v_width]
+        gate = proj[:, self.q_width + self.k_width + self.v_width :] if self.head_gate else None
+        if self.position is not None:
+            self.position.apply(q, k, ctx)
+        if cache.write:
+            kn.kv_store(k, v, self.kv_heads, self.key_dim, self.value_dim, ctx.row_pos, ctx.row_seq, ctx.seq_slot,
+                        cache.block_table, cache.k, cache.v, cache.block_size)
+        att = ctx.ws.alloc((rows, self.o_width), ctx.dtype)
+        kn.sink_attention(q, att, self.heads, self.kv_heads, self.key_dim, self.value_dim, ctx.row_pos, ctx.row_seq,
+                          ctx.seq_slot, cache.block_table, cache.k, cache.v, cache.block_size, self.scale,
+                          window=self.window, keep_first=self.keep_first, sink=self.sink, gate=gate,
+                          decode=ctx.decode)
+        if out is None:
+            out = ctx.ws.alloc((rows, self.width), torch.float32)
+        project(kn, ctx, att, self.w_o, out)
+        return out

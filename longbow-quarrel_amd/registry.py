@@ -1,4 +1,4 @@
-"""One registry from the architecture's name (config.json's `architectures[0]`)
+"""One registry from the architecture's name (config.json's `architectures[0]`, or its `architecture`)
 to its typed configuration and the function that turns it into a `ModelSpec`.
 
 The reference keeps a name -> creator map too (internal/engine/types_base.go:23-39),
@@ -26,8 +26,11 @@ def registered_architectures() -> List[str]:
 
 def architecture_of(config_dict: Dict[str, Any]) -> str:
     archs = config_dict.get("architectures")
+    if archs is None and isinstance(config_dict.get("architecture"), str):
+        return config_dict["architecture"]  # some designs name themselves with one string
     if not archs or not isinstance(archs, list) or not isinstance(archs[0], str):
-        raise ConfigError("config.json: 'architectures' must be a list that names the model class")
+        raise ConfigError("config.json: 'architectures' must be a list that names the model class "
+                          "(or 'architecture' a string)")
     return archs[0]
 
 

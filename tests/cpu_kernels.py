@@ -25,10 +25,10 @@ class CpuKernels:
     def use_stream(self, stream) -> None:
         pass
 
-    def embed(self, table, tokens, out):
+    def embed(self, table, tokens, out, scale=1.0):
         t = tokens[: out.shape[0]].long()
         known = (t >= 0) & (t < table.shape[0])  # no row of the table: zeros, as the library does
-        out.copy_(table[t.clamp(0, table.shape[0] - 1)].float() * known[:, None])
+        out.copy_(table[t.clamp(0, table.shape[0] - 1)].float() * known[:, None] * scale)
 
     @staticmethod
     def _whole(delta, like):
@@ -129,6 +129,123 @@ class CpuKernels:
                 s = (kk[:, g] @ qv) * scale
                 pr = torch.softmax(s, dim=0)
                 out[r, h * head_dim : (h + 1) * head_dim] = (pr[:, None] * vv[:, g]).sum(0).to(out.dtype)
+
+    # ---- the kernels of the recurrent mixers, the windowed attention with a sink and their norms ----
+    def dynamic_tanh(self, x, weight, bias, alpha, out, delta=None, delta_scale=1.0):
+        if delta is not None:
+            x += self._whole(delta, x) * delta_scale
+        out.copy_((torch.tanh(x * alpha) * weight + bias).to(out.dtype))
+
+    def add_scaled(self, x, delta, scale):
+        x += self._whole(delta, x) * scale
+
+    def glu(self, gate_up, out, activation):
+        inner = out.shape[1]
+        g, u = gate_up[:, :inner].float(), gate_up[:, inner:].float()
+        if activation == "relu":
+            a = torch.clamp(g, min=0)
+        elif activation == "silu":
+            a = g / (1 + torch.exp(-g))
+        elif activation == "gelu_tanh":
+            a = 0.5 * g * (1 + torch.tanh(math.sqrt(2 / math.pi) * (g + 0.044715 * g * g * g)))
+        else:
+            raise ValueError(activation)
+        out.copy_((a * u).to(out.dtype))
+
+    def kv_store(self, k, v, kv_heads, key_dim, value_dim, row_pos, row_seq, seq_slot, block_table, kcache, vcache,
+                 block_size):
+        for r in range(k.shape[0]):
+            p = int(row_pos[r])
+            blk = int(block_table[int(seq_slot[int(row_seq[r])]), p // block_size])
+            kcache[blk, :, p % block_size, :] = k[r].reshape(kv_heads, key_dim)
+            vcache[blk, :, :, p % block_size] = v[r].reshape(kv_heads, value_dim)
+
+    def sink_attention(self, q, out, heads, kv_heads, key_dim, value_dim, row_pos, row_seq, seq_slot, block_table,
+                       kcache, vcache, block_size, scale, window=0, keep_first=0, sink=True, gate=None, decode=False):
+        for r in range(q.shape[0]):
+            p = int(row_pos[r])
+            slot = int(seq_slot[int(row_seq[r])])
+            lo = p - window + 1 if (window > 0 and p >= window) else 0
+            ts = [t for t in range(p + 1) if t >= lo or t < keep_first]
+            kk = torch.stack([kcache[int(block_table[slot, t // block_size]), :, t % block_size, :] for t in ts]).float()
+            vv = torch.stack([vcache[int(block_table[slot, t // block_size]), :, :, t % block_size] for t in ts]).float()
+            for h in range(heads):
+                g = h // (heads // kv_heads)
+                s = (kk[:, g] @ q[r, h * key_dim : (h + 1) * key_dim].float()) * scale
+                m = torch.clamp(s.max(), min=0.0) if sink else s.max()
+                e = torch.exp(s - m)
+                denom = e.sum() + (torch.exp(-m) if sink else 0.0)
+                o = (e[:, None] * vv[:, g]).sum(0) / denom
+                if gate is not None:
+                    o = o * torch.sigmoid(gate[r, h].float())
+                out[r, h * value_dim : (h + 1) * value_dim] = o.to(out.dtype)
+
+    def causal_conv(self, x, weight, bias, state, out, row_pos, row_seq, seq_slot, seq_start, seq_len, cu_rows, batch,
+                    activation="silu"):
+        taps = weight.shape[1]
+        for b in range(batch):
+            r0, r1 = int(cu_rows[b]), int(cu_rows[b + 1])
+            slot = int(seq_slot[b])
+            hist = torch.cat([state[slot][: taps - 1], x[r0:r1].float()], 0) if taps > 1 else x[r0:r1].float()
+            y = torch.zeros((r1 - r0, x.shape[1]))
+            for j in range(taps):
+                y += hist[j : j + (r1 - r0)] * weight[:, j]
+            if bias is not None:
+                y += bias
+            if activation == "silu":
+                y = y / (1 + torch.exp(-y))
+            out[r0:r1] = y.to(out.dtype)
+            if taps > 1:
+                state[slot][: taps - 1] = hist[hist.shape[0] - (taps - 1) :]
+
+    def ssd_scan(self, x, b_in, c_in, dt, dt_bias, a_log, d_skip, state, y, heads, head_dim, n_state, groups, seq_slot,
+                 cu_rows, batch):
+        for b in range(batch):
+            r0, r1 = int(cu_rows[b]), int(cu_rows[b + 1])
+            s = state[int(seq_slot[b])]  # [heads, head_dim, n_state]
+            for r in range(r0, r1):
+                step = torch.nn.functional.softplus(dt[r].float() + dt_bias, threshold=1e9)
+                decay = torch.exp(-torch.exp(a_log) * step)
+                xr = x[r].float().reshape(heads, head_dim)
+                br = b_in[r].float().reshape(groups, n_state).repeat_interleave(heads // groups, 0)
+                cr = c_in[r].float().reshape(groups, n_state).repeat_interleave(heads // groups, 0)
+                s.mul_(decay[:, None, None]).add_(step[:, None, None] * xr[:, :, None] * br[:, None, :])
+                y[r] = ((s * cr[:, None, :]).sum(-1) + d_skip[:, None] * xr).reshape(-1)
+
+    def delta_scan(self, q, k, v, beta, a, dt_bias, a_log, state, out, heads, kv_heads, key_dim, value_dim, q_scale,
+                   unit_eps, seq_slot, cu_rows, batch):
+        rep = heads // kv_heads
+        for b in range(batch):
+            r0, r1 = int(cu_rows[b]), int(cu_rows[b + 1])
+            s = state[int(seq_slot[b])]  # [heads, value_dim, key_dim]
+            for r in range(r0, r1):
+                qr = q[r].float().reshape(kv_heads, key_dim)
+                kr = k[r].float().reshape(kv_heads, key_dim)
+                qr = (qr / torch.sqrt((qr * qr).sum(-1, keepdim=True) + unit_eps) * q_scale).repeat_interleave(rep, 0)
+                kr = (kr / torch.sqrt((kr * kr).sum(-1, keepdim=True) + unit_eps)).repeat_interleave(rep, 0)
+                vr = v[r].float().reshape(heads, value_dim)
+                bt = torch.sigmoid(beta[r].float())
+                g = torch.exp(-torch.exp(a_log) * torch.nn.functional.softplus(a[r].float() + dt_bias, threshold=1e9))
+                s.mul_(g[:, None, None])
+                u = bt[:, None] * (vr - (s * kr[:, None, :]).sum(-1))
+                s.add_(u[:, :, None] * kr[:, None, :])
+                out[r] = (s * qr[:, None, :]).sum(-1).reshape(-1)
+
+    def gated_rmsnorm(self, y, z, weight, eps, group, out, gate_first=True):
+        rows, n = y.shape
+        zf = z.float()
+        gate = zf / (1 + torch.exp(-zf))
+        v = y.float() * gate if gate_first else y.float()
+        v = v.reshape(rows, n // group, group)
+        v = (v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps)).reshape(rows, n)
+        v = v * (weight if weight.numel() == n else weight.repeat(n // weight.numel()))
+        out.copy_((v if gate_first else v * gate).to(out.dtype))
+
+    def rmsnorm_mean(self, stack, weights, eps, out):
+        acc = torch.zeros_like(out)
+        for t, w in zip(stack, weights):
+            acc += t / torch.sqrt((t * t).mean(-1, keepdim=True) + eps) * w
+        out.copy_(acc / len(weights))
 
     # greedy sampling and the upkeep of a decoding batch's arrays, so that the generation loop runs here too
     def argmax(self, logits, out, scratch=None, seq_slot=None, recent=None, recent_n=None):
