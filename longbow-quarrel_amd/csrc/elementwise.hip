@@ -12,7 +12,7 @@
 // slabs of 64 elements side by side: element k of row n lies at (n / 8) 8 D + (k / 64) 512 + (n % 8) 64 + k % 64.
 template <typename T>
 __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict__ tokens,
-                             float* __restrict__ out, int D, int vocab, int packed) {
+                             float* __restrict__ out, int D, int vocab, int packed, float scale) {
   const int r = blockIdx.x;
   const long long tok = tokens[r];
   const bool known = tok >= 0 && tok < vocab;
@@ -20,7 +20,7 @@ __global__ void embed_kernel(const T* __restrict__ table, const int* __restrict_
   const T* src = packed ? table + (row >> 3) * 8 * (long long)D + (row & 7) * 64 : table + row * (long long)D;
   float* dst = out + (long long)r * D;
   for (int j = threadIdx.x; j < D; j += blockDim.x)
-    dst[j] = known ? to_f32(src[packed ? ((j >> 6) << 9) + (j & 63) : j]) : 0.0f;
+    dst[j] = known ? to_f32(src[packed ? ((j >> 6) << 9) + (j & 63) : j]) * scale : 0.0f;
 }
 
 // A bfloat16 row of a width that is a multiple of 8, 16 bytes a lane and load: all of a thread's loads are on
@@ -31,7 +31,7 @@ typedef float embed_f32x4 __attribute__((ext_vector_type(4)));
 template <int PER_THREAD>
 __global__ __launch_bounds__(256) void embed_bf16_vec_kernel(const bf16_t* __restrict__ table,
                                                              const int* __restrict__ tokens, float* __restrict__ out,
-                                                             int D, int vocab, int packed) {
+                                                             int D, int vocab, int packed, float scale) {
   const int r = blockIdx.x;
   const long long tok = tokens[r];
   const bool known = tok >= 0 && tok < vocab;
@@ -51,34 +51,35 @@ __global__ __launch_bounds__(256) void embed_bf16_vec_kernel(const bf16_t* __res
   for (int i = 0; i < PER_THREAD; ++i) {
     const int c = threadIdx.x + i * 256;
     if (c < chunks) {
-      dst[2 * c] = (embed_f32x4){__uint_as_float(v[i][0] << 16), __uint_as_float(v[i][0] & 0xffff0000u),
-                                 __uint_as_float(v[i][1] << 16), __uint_as_float(v[i][1] & 0xffff0000u)};
-      dst[2 * c + 1] = (embed_f32x4){__uint_as_float(v[i][2] << 16), __uint_as_float(v[i][2] & 0xffff0000u),
-                                     __uint_as_float(v[i][3] << 16), __uint_as_float(v[i][3] & 0xffff0000u)};
+      dst[2 * c] = (embed_f32x4){__uint_as_float(v[i][0] << 16) * scale, __uint_as_float(v[i][0] & 0xffff0000u) * scale,
+                                 __uint_as_float(v[i][1] << 16) * scale, __uint_as_float(v[i][1] & 0xffff0000u) * scale};
+      dst[2 * c + 1] = (embed_f32x4){__uint_as_float(v[i][2] << 16) * scale, __uint_as_float(v[i][2] & 0xffff0000u) * scale,
+                                     __uint_as_float(v[i][3] << 16) * scale, __uint_as_float(v[i][3] & 0xffff0000u) * scale};
     }
   }
 }
 
+// out[r, :] = scale * table[tokens[r], :] (a model's own constant; 1 for most)
 extern "C" int lq_embed(const void* table, int table_dtype, const int* tokens, float* out, int rows,
-                        int D, int vocab, int packed, hipStream_t stream) {
+                        int D, int vocab, int packed, float scale, hipStream_t stream) {
   LQ_REQUIRE(rows > 0 && D > 0 && vocab > 0, "embed: rows %d, width %d and table rows %d must be positive", rows, D, vocab);
   LQ_REQUIRE(!packed || (D % 64 == 0 && vocab % 8 == 0), "embed: a packed table has rows in eights and a width in 64s");
   const int threads = D >= 1024 ? 256 : 64;
   if (table_dtype == LQ_BF16 && D % 8 == 0 && D >= 2048 && D <= 8 * 256 * 8 && (uintptr_t)table % 16 == 0 &&
       (uintptr_t)out % 16 == 0) {
     if (D <= 8 * 256 * 2)
-      embed_bf16_vec_kernel<2><<<rows, 256, 0, stream>>>((const bf16_t*)table, tokens, out, D, vocab, packed);
+      embed_bf16_vec_kernel<2><<<rows, 256, 0, stream>>>((const bf16_t*)table, tokens, out, D, vocab, packed, scale);
     else if (D <= 8 * 256 * 4)
-      embed_bf16_vec_kernel<4><<<rows, 256, 0, stream>>>((const bf16_t*)table, tokens, out, D, vocab, packed);
+      embed_bf16_vec_kernel<4><<<rows, 256, 0, stream>>>((const bf16_t*)table, tokens, out, D, vocab, packed, scale);
     else
-      embed_bf16_vec_kernel<8><<<rows, 256, 0, stream>>>((const bf16_t*)table, tokens, out, D, vocab, packed);
+      embed_bf16_vec_kernel<8><<<rows, 256, 0, stream>>>((const bf16_t*)table, tokens, out, D, vocab, packed, scale);
     LQ_CHECK_LAUNCH("embed");
     return 0;
   }
   if (table_dtype == LQ_F32)
-    embed_kernel<float><<<rows, threads, 0, stream>>>((const float*)table, tokens, out, D, vocab, packed);
+    embed_kernel<float><<<rows, threads, 0, stream>>>((const float*)table, tokens, out, D, vocab, packed, scale);
   else if (table_dtype == LQ_BF16)
-    embed_kernel<bf16_t><<<rows, threads, 0, stream>>>((const bf16_t*)table, tokens, out, D, vocab, packed);
+    embed_kernel<bf16_t><<<rows, threads, 0, stream>>>((const bf16_t*)table, tokens, out, D, vocab, packed, scale);
   else
     LQ_REQUIRE(false, "embed: unknown table dtype %d", table_dtype);
   LQ_CHECK_LAUNCH("embed");

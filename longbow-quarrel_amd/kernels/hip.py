@@ -20,7 +20,7 @@ from .. import build as _build
 from .dry import query
 
 F32, BF16 = 0, 1
-ABI_VERSION = 5  # lq_abi_version() of the library these wrappers were written for
+ABI_VERSION = 6  # lq_abi_version() of the library these wrappers were written for
 _DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
 
 
@@ -224,8 +224,8 @@ class HipKernels:
         self._check(self.lib.lq_pack_weight(_ptr(w), _ptr(out), c_int(n), c_int(k), self.stream))
         return PackedWeight(out, n, k)
 
-    def embed(self, table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor) -> None:
-        """out[r, :] = float32(table[tokens[r], :]); zeros where tokens[r] is no row of the table"""
+    def embed(self, table: torch.Tensor, tokens: torch.Tensor, out: torch.Tensor, scale: float = 1.0) -> None:
+        """out[r, :] = scale * float32(table[tokens[r], :]); zeros where tokens[r] is no row of the table"""
         self._dev(table, tokens, out)
         rows, width = out.shape
         self._i32(tokens, "embed tokens", rows)
@@ -235,7 +235,7 @@ class HipKernels:
             raise KernelLibraryError(f"embed: table {tuple(table.shape)} does not match width {width}")
         self._check(self.lib.lq_embed(_ptr(table), c_int(_code(table)), _ptr(tokens), _ptr(out),
                                       c_int(rows), c_int(width), c_int(table.shape[0]), c_int(_packed(table)),
-                                      self.stream))
+                                      c_float(scale), self.stream))
 
     @staticmethod
     def _pieces(delta: Optional[torch.Tensor], like: torch.Tensor, what: str):
@@ -665,6 +665,227 @@ class HipKernels:
                 tickets.zero_()
             finally:
                 raise KernelLibraryError(message)
+
+    # ------------------------------------------------------------------ windowed attention with a sink
+    def kv_store(self, k: torch.Tensor, v: torch.Tensor, kv_heads: int, key_dim: int, value_dim: int,
+                 row_pos: torch.Tensor, row_seq: torch.Tensor, seq_slot: torch.Tensor, block_table: torch.Tensor,
+                 kcache: torch.Tensor, vcache: torch.Tensor, block_size: int) -> None:
+        """k [rows, kv_heads * key_dim] and v [rows, kv_heads * value_dim] go into the paged cache as they are, at
+        the rows' positions (K [blocks, kv_heads, block_size, key_dim], V [blocks, kv_heads, value_dim, block_size])."""
+        self._dev(k, v, row_pos, row_seq, seq_slot, block_table, kcache, vcache)
+        rows = k.shape[0]
+        self._i32(row_pos, "row_pos", rows)
+        self._i32(row_seq, "row_seq", rows)
+        self._check_paged(kcache, vcache, kv_heads, key_dim, value_dim, block_size, block_table, seq_slot, "kv_store")
+        if v.shape[0] != rows or k.shape[1] != kv_heads * key_dim or v.shape[1] != kv_heads * value_dim \
+                or k.dtype != kcache.dtype or v.dtype != kcache.dtype:
+            raise KernelLibraryError("kv_store: k / v do not match the rows, the sizes or the cache's dtype")
+        self._check(self.lib.lq_kv_store(
+            _ptr(k), c_int(self._rows2d(k, "k")), _ptr(v), c_int(self._rows2d(v, "v")), c_int(_code(k)), c_int(rows),
+            c_int(kv_heads), c_int(key_dim), c_int(value_dim), _ptr(row_pos), _ptr(row_seq), _ptr(seq_slot),
+            _ptr(block_table), c_int(int(block_table.stride(0))), _ptr(kcache), _ptr(vcache), c_int(block_size),
+            self.stream))
+
+    @staticmethod
+    def _check_paged(kcache, vcache, kv_heads, key_dim, value_dim, block_size, block_table, seq_slot, what) -> None:
+        nb = kcache.shape[0]
+        if tuple(kcache.shape) != (nb, kv_heads, block_size, key_dim) or \
+                tuple(vcache.shape) != (nb, kv_heads, value_dim, block_size) or kcache.dtype != vcache.dtype or \
+                not kcache.is_contiguous() or not vcache.is_contiguous():
+            raise KernelLibraryError(f"{what}: cache tensors do not have the paged layout")
+        if seq_slot.dtype != torch.int32 or block_table.dtype != torch.int32 or block_table.dim() != 2:
+            raise KernelLibraryError(f"{what}: seq_slot and block_table must be int32 (table 2-D)")
+
+    def sink_attention(self, q: torch.Tensor, out: torch.Tensor, heads: int, kv_heads: int, key_dim: int,
+                       value_dim: int, row_pos: torch.Tensor, row_seq: torch.Tensor, seq_slot: torch.Tensor,
+                       block_table: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, block_size: int,
+                       scale: float, window: int = 0, keep_first: int = 0, sink: bool = True,
+                       gate: Optional[torch.Tensor] = None, decode: bool = False) -> None:
+        """Attention of the step's rows over their slots' cached keys: row at position p sees t <= p with
+        p - t < window (0: all) or t < keep_first; with `sink` the softmax's denominator has one more term e^0;
+        `gate` [rows, heads]: every head's result times the sigmoid of its entry.  Scores and probabilities
+        are 32-bit.  out [rows, heads * value_dim] in the dtype of q and the cache."""
+        self._dev(q, out, gate, row_pos, row_seq, seq_slot, block_table, kcache, vcache)
+        rows, batch = q.shape[0], seq_slot.numel()
+        self._i32(row_pos, "row_pos", rows)
+        self._i32(row_seq, "row_seq", rows)
+        self._check_paged(kcache, vcache, kv_heads, key_dim, value_dim, block_size, block_table, seq_slot, "sink_attention")
+        if q.shape[1] != heads * key_dim or tuple(out.shape) != (rows, heads * value_dim) or q.dtype != out.dtype \
+                or q.dtype != kcache.dtype:
+            raise KernelLibraryError("sink_attention: q / out do not match the rows, the sizes or the cache's dtype")
+        if gate is not None and (tuple(gate.shape) != (rows, heads) or gate.dtype != q.dtype):
+            raise KernelLibraryError("sink_attention: the gate is [rows, heads] in the dtype of q")
+        if decode and rows != batch:
+            raise KernelLibraryError("sink_attention: decode means one row per sequence")
+        self._check(self.lib.lq_sink_attention(
+            _ptr(q), c_int(self._rows2d(q, "q")), _ptr(out), c_int(self._rows2d(out, "out")), _ptr(gate),
+            c_int(0 if gate is None else self._rows2d(gate, "gate")), c_int(_code(q)), c_int(rows), c_int(batch),
+            c_int(heads), c_int(kv_heads), c_int(key_dim), c_int(value_dim), _ptr(row_pos), _ptr(row_seq),
+            _ptr(seq_slot), _ptr(block_table), c_int(int(block_table.stride(0))), _ptr(kcache), _ptr(vcache),
+            c_int(block_size), c_float(scale), c_int(window), c_int(keep_first), c_int(1 if sink else 0),
+            c_int(1 if self.force_generic else 0), self.stream))
+
+    # ------------------------------------------------------------------ recurrent mixers and what surrounds them
+    _ACTIVATIONS = {"none": 0, "silu": 1, "relu": 2, "gelu_tanh": 3}
+
+    @staticmethod
+    def _f32(t: torch.Tensor, what: str, n: Optional[int] = None) -> None:
+        if t.dtype != torch.float32 or not t.is_cuda or (n is not None and (t.numel() != n or not t.is_contiguous())):
+            raise KernelLibraryError(f"{what}: a float32 tensor on the GPU" + (f" of {n} entries" if n is not None else ""))
+
+    def dynamic_tanh(self, x: torch.Tensor, weight: torch.Tensor, bias: torch.Tensor, alpha: torch.Tensor,
+                     out: torch.Tensor, delta: Optional[torch.Tensor] = None, delta_scale: float = 1.0) -> None:
+        """(x += delta_scale * delta;) out = tanh(alpha x) weight + bias; x float32, alpha a tensor of one entry."""
+        rows, width, ldx = self._mat(x, "dynamic_tanh: x")
+        self._f32(x, "dynamic_tanh: x")
+        self._f32(weight, "dynamic_tanh: weight", width)
+        self._f32(bias, "dynamic_tanh: bias", width)
+        self._f32(alpha, "dynamic_tanh: alpha", 1)
+        pieces, stride = self._pieces(delta, x, "dynamic_tanh")
+        if delta is not None:
+            self._f32(delta, "dynamic_tanh: delta")
+        if not x.is_contiguous() or not out.is_contiguous() or tuple(out.shape) != (rows, width) or not out.is_cuda:
+            raise KernelLibraryError("dynamic_tanh: x and out must be dense and of one shape")
+        self._check(self.lib.lq_dynamic_tanh(_ptr(x), _ptr(delta), c_int(pieces), c_longlong(stride),
+                                             c_float(delta_scale), _ptr(weight), _ptr(bias), _ptr(alpha), _ptr(out),
+                                             c_int(_code(out)), c_int(rows), c_int(width), self.stream))
+
+    def add_scaled(self, x: torch.Tensor, delta: torch.Tensor, scale: float) -> None:
+        """x += scale * delta (delta shaped like x, or a stack of pieces whose sum is meant); float32."""
+        self._f32(x, "add_scaled: x")
+        self._f32(delta, "add_scaled: delta")
+        pieces, stride = self._pieces(delta, x, "add_scaled")
+        if not x.is_contiguous():
+            raise KernelLibraryError("add_scaled: x must be dense")
+        self._check(self.lib.lq_add_scaled(_ptr(x), _ptr(delta), c_int(pieces), c_longlong(stride), c_float(scale),
+                                           c_longlong(x.numel()), self.stream))
+
+    def glu(self, gate_up: torch.Tensor, out: torch.Tensor, activation: str) -> None:
+        """out = act(gate) * up for gate_up [rows, 2 * inner] = [gate | up]; act: silu, relu or gelu_tanh."""
+        rows, two, ld = self._mat(gate_up, "glu: gate_up")
+        ro, inner, ldo = self._mat(out, "glu: out")
+        if ro != rows or two != 2 * inner or activation not in self._ACTIVATIONS or activation == "none":
+            raise KernelLibraryError(f"glu: gate_up {tuple(gate_up.shape)}, out {tuple(out.shape)}, activation {activation!r}")
+        self._check(self.lib.lq_glu(_ptr(gate_up), c_int(_code(gate_up)), c_int(ld), _ptr(out), c_int(_code(out)),
+                                    c_int(ldo), c_int(rows), c_int(inner), c_int(self._ACTIVATIONS[activation]),
+                                    self.stream))
+
+    def causal_conv(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], state: torch.Tensor,
+                    out: torch.Tensor, row_pos: torch.Tensor, row_seq: torch.Tensor, seq_slot: torch.Tensor,
+                    seq_start: torch.Tensor, seq_len: torch.Tensor, cu_rows: torch.Tensor, batch: int,
+                    activation: str = "silu") -> None:
+        """out[t, c] = act(bias[c] + sum_j weight[c, j] x[t - (taps - 1) + j, c]) along every sequence of the step;
+        what lies before the step's rows comes from state [slots, taps - 1, channels] (a sequence's last inputs,
+        zeros at its start), which is then moved on to the step's end.  All float32."""
+        rows, ch, ldx = self._mat(x, "causal_conv: x")
+        ro, co, ldo = self._mat(out, "causal_conv: out")
+        taps = weight.shape[1] if weight.dim() == 2 else 0
+        for t, what in ((x, "x"), (out, "out"), (state, "state")):
+            self._f32(t, "causal_conv: " + what)
+        self._f32(weight, "causal_conv: weight", ch * max(1, taps))
+        if bias is not None:
+            self._f32(bias, "causal_conv: bias", ch)
+        if (ro, co) != (rows, ch) or taps < 1 or state.dim() != 3 or tuple(state.shape[1:]) != (max(1, taps - 1), ch) \
+                or not state.is_contiguous() or activation not in self._ACTIVATIONS:
+            raise KernelLibraryError("causal_conv: x, out [rows, channels], weight [channels, taps], "
+                                     "state [slots, taps - 1, channels] do not fit")
+        self._i32(row_pos, "row_pos", rows)
+        self._i32(row_seq, "row_seq", rows)
+        self._i32(seq_slot, "seq_slot", batch)
+        self._i32(seq_start, "seq_start", batch)
+        self._i32(cu_rows, "cu_rows", batch + 1)
+        self._check(self.lib.lq_causal_conv(_ptr(x), c_int(ldx), _ptr(weight), _ptr(bias), _ptr(state), _ptr(out),
+                                            c_int(ldo), c_int(rows), c_int(ch), c_int(taps), _ptr(row_seq), _ptr(row_pos),
+                                            _ptr(seq_slot), _ptr(seq_start), _ptr(cu_rows), c_int(batch),
+                                            c_int(self._ACTIVATIONS[activation]), self.stream))
+
+    def ssd_scan(self, x: torch.Tensor, b_in: torch.Tensor, c_in: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor,
+                 a_log: torch.Tensor, d_skip: torch.Tensor, state: torch.Tensor, y: torch.Tensor, heads: int,
+                 head_dim: int, n_state: int, groups: int, seq_slot: torch.Tensor, cu_rows: torch.Tensor,
+                 batch: int) -> None:
+        """The Mamba-2 recurrence along every sequence of the step, token by token: with dt = softplus(dt + dt_bias),
+        S <- exp(-exp(a_log) dt) S + dt B x^T and y = S^T C + d_skip x per head; state [slots, heads, head_dim,
+        n_state] is read and left at the step's end.  All float32."""
+        rows = x.shape[0]
+        for t, what, cols in ((x, "x", heads * head_dim), (b_in, "B", groups * n_state), (c_in, "C", groups * n_state),
+                              (dt, "dt", heads), (y, "y", heads * head_dim)):
+            self._f32(t, "ssd_scan: " + what)
+            if self._mat(t, "ssd_scan: " + what)[:2] != (rows, cols):
+                raise KernelLibraryError(f"ssd_scan: {what} must be [{rows}, {cols}], found {tuple(t.shape)}")
+        for t, what in ((dt_bias, "dt_bias"), (a_log, "a_log"), (d_skip, "d_skip")):
+            self._f32(t, "ssd_scan: " + what, heads)
+        self._f32(state, "ssd_scan: state")
+        if state.dim() != 4 or tuple(state.shape[1:]) != (heads, head_dim, n_state) or not state.is_contiguous():
+            raise KernelLibraryError("ssd_scan: state must be dense [slots, heads, head_dim, n_state]")
+        self._i32(seq_slot, "seq_slot", batch)
+        self._i32(cu_rows, "cu_rows", batch + 1)
+        ld = self._rows2d
+        self._check(self.lib.lq_ssd_scan(_ptr(x), c_int(ld(x, "x")), _ptr(b_in), c_int(ld(b_in, "B")), _ptr(c_in),
+                                         c_int(ld(c_in, "C")), _ptr(dt), c_int(ld(dt, "dt")), _ptr(dt_bias), _ptr(a_log),
+                                         _ptr(d_skip), _ptr(state), _ptr(y), c_int(ld(y, "y")), c_int(heads),
+                                         c_int(head_dim), c_int(n_state), c_int(groups), _ptr(seq_slot), _ptr(cu_rows),
+                                         c_int(batch), self.stream))
+
+    def delta_scan(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, beta: torch.Tensor, a: torch.Tensor,
+                   dt_bias: torch.Tensor, a_log: torch.Tensor, state: torch.Tensor, out: torch.Tensor, heads: int,
+                   kv_heads: int, key_dim: int, value_dim: int, q_scale: float, unit_eps: float,
+                   seq_slot: torch.Tensor, cu_rows: torch.Tensor, batch: int) -> None:
+        """The gated delta rule along every sequence of the step, token by token: q and k made unit vectors per
+        head (x / sqrt(sum x^2 + unit_eps)), q times q_scale, beta = sigmoid(beta), g = exp(-exp(a_log)
+        softplus(a + dt_bias)); S <- g S, u = beta (v - S^T k), S <- S + k u^T, out = S^T q.  state [slots, heads,
+        value_dim, key_dim].  All float32."""
+        rows = q.shape[0]
+        for t, what, cols in ((q, "q", kv_heads * key_dim), (k, "k", kv_heads * key_dim), (v, "v", heads * value_dim),
+                              (beta, "beta", heads), (a, "a", heads), (out, "out", heads * value_dim)):
+            self._f32(t, "delta_scan: " + what)
+            if self._mat(t, "delta_scan: " + what)[:2] != (rows, cols):
+                raise KernelLibraryError(f"delta_scan: {what} must be [{rows}, {cols}], found {tuple(t.shape)}")
+        self._f32(dt_bias, "delta_scan: dt_bias", heads)
+        self._f32(a_log, "delta_scan: a_log", heads)
+        self._f32(state, "delta_scan: state")
+        if state.dim() != 4 or tuple(state.shape[1:]) != (heads, value_dim, key_dim) or not state.is_contiguous():
+            raise KernelLibraryError("delta_scan: state must be dense [slots, heads, value_dim, key_dim]")
+        self._i32(seq_slot, "seq_slot", batch)
+        self._i32(cu_rows, "cu_rows", batch + 1)
+        ld = self._rows2d
+        self._check(self.lib.lq_delta_scan(_ptr(q), c_int(ld(q, "q")), _ptr(k), c_int(ld(k, "k")), _ptr(v),
+                                           c_int(ld(v, "v")), _ptr(beta), c_int(ld(beta, "beta")), _ptr(a),
+                                           c_int(ld(a, "a")), _ptr(dt_bias), _ptr(a_log), _ptr(state), _ptr(out),
+                                           c_int(ld(out, "out")), c_int(heads), c_int(kv_heads), c_int(key_dim),
+                                           c_int(value_dim), c_float(q_scale), c_float(unit_eps), _ptr(seq_slot),
+                                           _ptr(cu_rows), c_int(batch), self.stream))
+
+    def gated_rmsnorm(self, y: torch.Tensor, z: torch.Tensor, weight: torch.Tensor, eps: float, group: int,
+                      out: torch.Tensor, gate_first: bool = True) -> None:
+        """RMS norm of y [rows, n] in parts of `group` columns, each by its own root mean square, with a gate
+        silu(z): gate_first: (y silu(z)) normed, times weight; else y normed, times weight, times silu(z).  The
+        weight has n entries, or fewer that repeat (one weight for every part)."""
+        rows, n, ldy = self._mat(y, "gated_rmsnorm: y")
+        rz, nz, ldz = self._mat(z, "gated_rmsnorm: z")
+        ro, no, ldo = self._mat(out, "gated_rmsnorm: out")
+        self._f32(y, "gated_rmsnorm: y")
+        self._f32(z, "gated_rmsnorm: z")
+        self._f32(weight, "gated_rmsnorm: weight", weight.numel())
+        if (rz, nz) != (rows, n) or (ro, no) != (rows, n) or group <= 0 or n % group:
+            raise KernelLibraryError("gated_rmsnorm: y, z and out must be [rows, n] with n a multiple of the group")
+        self._check(self.lib.lq_gated_rmsnorm(_ptr(y), c_int(ldy), _ptr(z), c_int(ldz), _ptr(weight),
+                                              c_int(weight.numel()), c_float(eps), c_int(group), _ptr(out),
+                                              c_int(_code(out)), c_int(ldo), c_int(rows), c_int(n),
+                                              c_int(1 if gate_first else 0), self.stream))
+
+    def rmsnorm_mean(self, stack: torch.Tensor, weights, eps: float, out: torch.Tensor) -> None:
+        """out = mean over i of stack[i] / rms(stack[i]) * weights[i], row by row; stack [n, rows, width] float32."""
+        self._f32(stack, "rmsnorm_mean: stack")
+        self._f32(out, "rmsnorm_mean: out")
+        if stack.dim() != 3 or not stack.is_contiguous() or not out.is_contiguous() \
+                or tuple(out.shape) != tuple(stack.shape[1:]) or len(weights) != stack.shape[0] or not 1 <= len(weights) <= 4:
+            raise KernelLibraryError("rmsnorm_mean: a dense stack [n, rows, width] of 1 to 4 branches, a weight for each")
+        n, rows, width = stack.shape
+        for w in weights:
+            self._f32(w, "rmsnorm_mean: weight", width)
+        ws = [_ptr(w) for w in weights] + [c_void_p(0)] * (4 - n)
+        self._check(self.lib.lq_rmsnorm_mean(_ptr(stack), c_int(n), *ws, c_float(eps), _ptr(out), c_int(rows),
+                                             c_int(width), self.stream))
 
     # ------------------------------------------------------------------ sampling
     @property
