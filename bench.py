@@ -22,6 +22,12 @@ seed) and then K decoding steps, all of it through the generation loop (`Generat
 prompts in portions of 8,192 rows, captured decoding steps); once with W steps untimed, then timed.
 `--shape 70b`: the 70B layer sizes, batch 8 from 1,024-token prompts, with batch 1 and a
 2,048-token prefill as points.
+
+`--design vafodra`: the hybrid design (windowed attention with a sink beside Mamba-2, and the gated delta rule) at
+layer sizes of a real model, beside the Llama shape of the same width, depth, feed-forward and vocabulary: for each
+of `--design-widths` a prefill of `--prefill-tokens` tokens and decoding at `--batch` from `--prompt-len`-token
+prompts (captured steps), then device time by operation for both (events around every kernel call).  One JSON line;
+the default run is not changed by it.
 """
 from __future__ import annotations
 
@@ -78,6 +84,100 @@ def prefill_flops(c, t: int) -> float:
     return c.num_hidden_layers * (linear + attention) + 2.0 * d * c.vocab_size
 
 
+def vafodra_config(width: int, layers: int, vocab: int) -> dict:
+    """Layer sizes of a real model for the hybrid design: per four layers three parallel ones (attention heads of
+    128 over a window of 1,024 that keeps 4 tokens; a state-space side as wide as the model with a state of 128) and
+    one gated delta layer; the feed-forward 3.5 times the width, as the Llama shape beside it."""
+    heads = width // 128
+    left = {"dim": 128, "vdim": 128, "heads": heads, "kv_heads": max(1, heads // 4),
+            "mask": {"size": 1024, "keep_first": 4}, "scale": 128 ** -0.5}
+    right = {"conv": 4, "groups": 8, "heads": width // 64, "norm_groups": 8, "state": 128, "vdim": 64}
+    delta = {"conv": 4, "dim": 128, "heads": heads, "kv_heads": max(1, heads // 2), "vdim": 128}
+    mlp = {"kind": "dense", "ff": width * 7 // 2}
+    made = [{"type": "delta", "mixer": delta, "mlp": mlp} if i % 4 == 3 else
+            {"type": "parallel", "mixer": {"left": left, "right": right}, "mlp": mlp} for i in range(layers)]
+    return {"architecture": "Vafodra", "embedding": {"scale": 1.0}, "layers": made, "norm": {"eps": 1e-5},
+            "residual_mult": 0.5, "vocab": vocab, "width": width}
+
+
+def design_run(args) -> int:
+    import torch
+
+    import longbow_quarrel_amd as lq
+    from longbow_quarrel_amd.engine import EngineBackend, StepEntry
+    from longbow_quarrel_amd.kernels.timed import TimedKernels
+
+    layers, vocab = args.layers or 8, 32000
+    batch, prompt_len, n_prefill = args.batch or 8, args.prompt_len or 512, args.prefill_tokens
+    gen = torch.Generator().manual_seed(1234)
+    results = []
+    for width in [int(w) for w in args.design_widths.split(",")]:
+        llama = dict(CONFIG_8B, hidden_size=width, intermediate_size=width * 7 // 2, num_hidden_layers=layers,
+                     num_attention_heads=width // 128, num_key_value_heads=max(1, width // 512), vocab_size=vocab)
+        for name, config in (("vafodra", lq.VafodraConfig.from_dict(vafodra_config(width, layers, vocab))),
+                             ("llama", lq.LlamaConfig.from_dict(llama))):
+            engine = lq.random_engine(config, seed=0, dtype=args.dtype, max_tokens=batch * 4096 + n_prefill + 64,
+                                      max_slots=batch + 1, max_sequence_tokens=max(4096, n_prefill))
+            prompt = lambda n: torch.randint(0, vocab, (n,), generator=gen).tolist()
+            times = []
+            for i in range(4):  # the first untimed
+                slot = engine.new_sequence()
+                torch.cuda.synchronize()
+                t = time.perf_counter()
+                engine.step([StepEntry(slot, prompt(n_prefill), [n_prefill - 1])])
+                torch.cuda.synchronize()
+                times.append(time.perf_counter() - t)
+                engine.release(slot)
+            prefill_ms = sorted(times[1:])[1] * 1e3
+            backend = EngineBackend(engine, lq.SamplingParams(temperature=0.0), use_graphs=True)
+            slots = [backend.new_sequence(r, [0]) for r in range(batch)]
+            toks = backend.prefill(slots, [prompt(prompt_len) for _ in range(batch)])
+            for i in range(args.warmup):
+                backend.expect_more(i + 1 < args.warmup)
+                toks = backend.decode(slots, toks, False)
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            for i in range(args.steps):
+                backend.expect_more(i + 1 < args.steps)
+                toks = backend.decode(slots, toks, False)
+            torch.cuda.synchronize()
+            step_ms = (time.perf_counter() - t) / args.steps * 1e3
+            for s in slots:
+                backend.release(s)
+            backend.close()
+            # device time by operation, steps run directly
+            timed = TimedKernels(engine.kernels)
+            engine.kernels = timed
+            by_op = {}
+            slots = [engine.new_sequence() for _ in range(batch)]
+            engine.step([StepEntry(slots[0], prompt(n_prefill), [n_prefill - 1])])
+            engine.release(slots[0])
+            slots[0] = engine.new_sequence()
+            timed.reset()
+            engine.step([StepEntry(slots[0], prompt(n_prefill), [n_prefill - 1])])
+            by_op["prefill"] = {op: round(ms / layers * 1e3, 1) for op, (calls, ms) in timed.report().items()}
+            engine.release(slots[0])
+            slots[0] = engine.new_sequence()
+            engine.step([StepEntry(s, prompt(prompt_len), [prompt_len - 1]) for s in slots])
+            engine.step([StepEntry(s, [1], [0]) for s in slots])
+            timed.reset()
+            for _ in range(8):
+                engine.step([StepEntry(s, [1], [0]) for s in slots])
+            by_op["decode"] = {op: round(ms / 8 / layers * 1e3, 1) for op, (calls, ms) in timed.report().items()}
+            line = {"design": name, "width": width, "layers": layers, "prefill_tokens": n_prefill,
+                    "prefill_ms": round(prefill_ms, 3), "prefill_tok_s": round(n_prefill / prefill_ms * 1e3, 1),
+                    "decode_batch": batch, "decode_ms_per_step": round(step_ms, 4),
+                    "decode_tok_s": round(batch / step_ms * 1e3, 1), "us_per_layer_by_operation": by_op}
+            print(f"[bench] {json.dumps(line)}", file=sys.stderr, flush=True)
+            results.append(line)
+            del engine, backend, timed
+            torch.cuda.empty_cache()
+    print(json.dumps({"metric": "prefill and decode tok/s of the Vafodra design beside the Llama shape of equal size",
+                      "dtype": args.dtype, "data": "synthetic: random weights from a seed, uniform random token ids",
+                      "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "results": results}), flush=True)
+    return 0
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -102,10 +202,15 @@ def main() -> int:
                     help="float32: the true 32-bit path (use --layers with the larger shapes)")
     ap.add_argument("--context", type=int, default=0,
                     help="tokens a sequence may hold (default: the shape's 8192); for decoding over longer prompts")
+    ap.add_argument("--design", choices=["vafodra"], default=None,
+                    help="measure this design beside the Llama shape of equal size instead of the default workload")
+    ap.add_argument("--design-widths", default="2048,4096", help="model widths of --design, with commas between them")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this library runs on one GPU; --gpus {args.gpus} is not supported")
         return 2
+    if args.design:
+        return design_run(args)
     through_loop = args.shape == "1b"  # the workload with unequal prompts runs through the generation loop
     args.batch = args.batch or (16 if args.shape == "1b" else 8)
     args.prompt_len = args.prompt_len or {"8b": 512, "1b": 64, "70b": 1024}[args.shape]
