@@ -40,18 +40,31 @@ struct SinkArgs {
 
 constexpr int MAX_KD = 256;
 
-// A wavefront takes up to 16 consecutive rows of the step and one query head.  For every sequence with rows in
-// the tile it walks the chunks that any of these rows sees; rows of other sequences and keys that a row does not
-// see take part with weight zero.  Per chunk: S^T = K . Q^T (16 keys by 16 rows a product), the softmax of every
-// row over its 64 scores, O += P . V with the probabilities straight from the registers of the scores.  A lane
-// (c, g) keeps the part of row c's query that it multiplies (dimensions 16 s + 4 g .. + 3 of every slab s) in LDS,
-// where only it reads it: the key size is then a loop bound and no template parameter.
+// A workgroup of SPLIT wavefronts takes up to 16 consecutive rows of the step and one query head.  For every
+// sequence with rows in the tile it walks the chunks that any of these rows sees, wavefront w the chunks whose
+// number (position / 64) is w modulo SPLIT; rows of other sequences and keys that a row does not see take part with
+// weight zero.  Per chunk: S^T = K . Q^T (16 keys by 16 rows a product), the softmax of every row over its 64
+// scores, O += P . V with the probabilities straight from the registers of the scores.  At the end the wavefronts'
+// partial results (maximum, sum, weighted values) meet in LDS and are merged in the order of the wavefronts.  Which
+// wavefront takes which chunk follows from positions alone, so a row's sums are the same in every launch.
+// A lane (c, g) keeps the part of row c's query that it multiplies (dimensions 16 s + 4 g .. + 3 of every slab s) in
+// LDS, where only it reads it: the key size is then a loop bound and no template parameter.  bfloat16 keys and
+// queries are multiplied as they are (v_mfma_f32_16x16x16_bf16: the products are exact, the sums 32-bit); the
+// probabilities stay 32-bit and meet the widened values in the 32-bit product.
+constexpr int SPLIT = 4;
+typedef short bf16x4 __attribute__((ext_vector_type(4)));
+
 template <typename T, int HSV>  // HSV: value size / 16
-__global__ __launch_bounds__(64) void sink_tiles_kernel(const T* __restrict__ q, T* __restrict__ out,
-                                                        const T* __restrict__ gate, const T* __restrict__ kcache,
-                                                        const T* __restrict__ vcache, SinkArgs a) {
-  __shared__ float qs[16 * 4 * (MAX_KD / 4 + 4)];  // [g][c][slab][4], a lane's own run padded against bank clashes
-  const int lane = threadIdx.x, c = lane & 15, g = lane >> 4;
+__global__ __launch_bounds__(64 * SPLIT) void sink_tiles_kernel(const T* __restrict__ q, T* __restrict__ out,
+                                                                const T* __restrict__ gate,
+                                                                const T* __restrict__ kcache,
+                                                                const T* __restrict__ vcache, SinkArgs a) {
+  constexpr bool HALF = sizeof(T) == 2;
+  constexpr int QROW = MAX_KD / 4 + 4;             // a lane's own run of q, padded against bank clashes
+  constexpr int PART = 64 * (HSV * 4) + 32;        // a wavefront's partial result: o of every lane, then m and l of 16 rows
+  constexpr int LDS_FLOATS = 64 * QROW > (SPLIT - 1) * PART ? 64 * QROW : (SPLIT - 1) * PART;
+  __shared__ float smem[LDS_FLOATS];               // first the queries, at the end the partial results
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, c = lane & 15, g = lane >> 4;
   const int h = blockIdx.y, kvh = h / (a.nh / a.nkv);
   const int r0 = blockIdx.x * a.rows_per_tile;
   const int n_rows = min(a.rows_per_tile, a.rows - r0);
@@ -59,11 +72,19 @@ __global__ __launch_bounds__(64) void sink_tiles_kernel(const T* __restrict__ q,
   const int my_row = r0 + min(c, n_rows - 1);
   const int my_pos = a.row_pos[my_row], my_seq = a.row_seq[my_row];
   const int my_lo = (a.window > 0 && my_pos >= a.window) ? my_pos - a.window + 1 : 0;
-  float* myq = qs + (g * 16 + c) * (MAX_KD / 4 + 4);
-  for (int sl = 0; sl < HS; ++sl)
-    *(f32x4*)(myq + 4 * sl) = ld4(q + (long long)my_row * a.ldq + h * a.KD + sl * 16 + 4 * g);
+  float* myq = smem + (g * 16 + c) * QROW;
+  if (wave == 0) {
+    for (int sl = 0; sl < HS; ++sl) {
+      const T* src = q + (long long)my_row * a.ldq + h * a.KD + sl * 16 + 4 * g;
+      if constexpr (HALF) *(uint2*)(myq + 4 * sl) = *(const uint2*)src;
+      else *(f32x4*)(myq + 4 * sl) = ld4(src);
+    }
+  }
+  __syncthreads();
 
-  float m = a.sink ? 0.f : -INFINITY, l = a.sink ? 1.f : 0.f;
+  // the sink is one more key of score 0 without a value: the first wavefront starts from it
+  const bool with_sink = a.sink && wave == 0;
+  float m = with_sink ? 0.f : -INFINITY, l = with_sink ? 1.f : 0.f;
   f32x4 o[HSV];  // o[dt][e]: row 4 g + e of the tile, value dimension 16 dt + c
 #pragma unroll
   for (int dt = 0; dt < HSV; ++dt) o[dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
@@ -86,70 +107,111 @@ __global__ __launch_bounds__(64) void sink_tiles_kernel(const T* __restrict__ q,
     const int kept_end = min(a.keep_first, wstart);  // kept keys that lie below that chunk
     int t0 = kept_end > 0 ? 0 : wstart;
     while (t0 <= pos_max) {
-      f32x4 st[4];  // st[kt][e]: score of key t0 + 16 kt + 4 g + e for row c
+      if (((t0 >> 6) & (SPLIT - 1)) == wave) {
+        f32x4 st[4];  // st[kt][e]: score of key t0 + 16 kt + 4 g + e for row c
 #pragma unroll
-      for (int kt = 0; kt < 4; ++kt) {
-        st[kt] = (f32x4){0.f, 0.f, 0.f, 0.f};
-        const int t = min(t0 + 16 * kt + c, pos_max);  // this lane's key as an operand row (clamped: finite, masked below)
-        const long long blk = table[t / BS];
-        const T* kr = kcache + ((blk * a.nkv + kvh) * BS + t % BS) * (long long)a.KD + 4 * g;
-        for (int sl = 0; sl < HS; ++sl) {
-          const f32x4 kv = ld4(kr + sl * 16);
-          const f32x4 qv = *(const f32x4*)(myq + 4 * sl);
+        for (int kt = 0; kt < 4; ++kt) {
+          st[kt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+          const int t = min(t0 + 16 * kt + c, pos_max);  // this lane's key as an operand row (clamped: finite, masked below)
+          const long long blk = table[t / BS];
+          const T* kr = kcache + ((blk * a.nkv + kvh) * BS + t % BS) * (long long)a.KD + 4 * g;
+          if constexpr (HALF) {
+            for (int sl = 0; sl < HS; ++sl) {
+              const uint2 kv = *(const uint2*)(kr + sl * 16);
+              const uint2 qv = *(const uint2*)(myq + 4 * sl);
+              st[kt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(__builtin_bit_cast(bf16x4, kv),
+                                                                 __builtin_bit_cast(bf16x4, qv), st[kt], 0, 0, 0);
+            }
+          } else {
+            for (int sl = 0; sl < HS; ++sl) {
+              const f32x4 kv = ld4(kr + sl * 16);
+              const f32x4 qv = *(const f32x4*)(myq + 4 * sl);
 #pragma unroll
-          for (int j = 0; j < 4; ++j) st[kt] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv[j], qv[j], st[kt], 0, 0, 0);
+              for (int j = 0; j < 4; ++j) st[kt] = __builtin_amdgcn_mfma_f32_16x16x4f32(kv[j], qv[j], st[kt], 0, 0, 0);
+            }
+          }
         }
-      }
-      float cmax = -INFINITY;
+        float cmax = -INFINITY;
 #pragma unroll
-      for (int kt = 0; kt < 4; ++kt)
+        for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const int t = t0 + 16 * kt + 4 * g + e;
-          const bool valid = mine && t <= my_pos && (t >= my_lo || t < a.keep_first);
-          st[kt][e] = valid ? st[kt][e] * a.scale : -INFINITY;
-          cmax = fmaxf(cmax, st[kt][e]);
-        }
-      cmax = fmaxf(cmax, __shfl_xor(cmax, 16, 64));
-      cmax = fmaxf(cmax, __shfl_xor(cmax, 32, 64));
-      const float m_new = fmaxf(m, cmax);
-      const bool none = m_new == -INFINITY;  // no key of this row so far and no sink: nothing changes
-      const float alpha = none ? 1.f : expf(m - m_new);
-      float psum = 0.f;
+          for (int e = 0; e < 4; ++e) {
+            const int t = t0 + 16 * kt + 4 * g + e;
+            const bool valid = mine && t <= my_pos && (t >= my_lo || t < a.keep_first);
+            st[kt][e] = valid ? st[kt][e] * a.scale : -INFINITY;
+            cmax = fmaxf(cmax, st[kt][e]);
+          }
+        cmax = fmaxf(cmax, __shfl_xor(cmax, 16, 64));
+        cmax = fmaxf(cmax, __shfl_xor(cmax, 32, 64));
+        const float m_new = fmaxf(m, cmax);
+        const bool none = m_new == -INFINITY;  // no key of this row so far and no sink: nothing changes
+        const float alpha = none ? 1.f : expf(m - m_new);
+        float psum = 0.f;
 #pragma unroll
-      for (int kt = 0; kt < 4; ++kt)
+        for (int kt = 0; kt < 4; ++kt)
 #pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          st[kt][e] = none ? 0.f : expf(st[kt][e] - m_new);
-          psum += st[kt][e];
-        }
-      psum += __shfl_xor(psum, 16, 64);
-      psum += __shfl_xor(psum, 32, 64);
-      l = l * alpha + psum;
-      m = m_new;
-      float a4[4];
+          for (int e = 0; e < 4; ++e) {
+            st[kt][e] = none ? 0.f : expf(st[kt][e] - m_new);
+            psum += st[kt][e];
+          }
+        psum += __shfl_xor(psum, 16, 64);
+        psum += __shfl_xor(psum, 32, 64);
+        l = l * alpha + psum;
+        m = m_new;
+        float a4[4];
 #pragma unroll
-      for (int e = 0; e < 4; ++e) a4[e] = __shfl(alpha, 4 * g + e, 64);
-#pragma unroll
-      for (int dt = 0; dt < HSV; ++dt)
-#pragma unroll
-        for (int e = 0; e < 4; ++e) o[dt][e] *= a4[e];
-#pragma unroll
-      for (int kt = 0; kt < 4; ++kt) {
-        // V^T of this lane's dimension 16 dt + c at keys t0 + 16 kt + 4 g .. + 3 (within one block)
-        const int t = min(t0 + 16 * kt + 4 * g, pos_max) & ~3;
-        const long long blk = table[t / BS];
-        const T* vr = vcache + ((blk * a.nkv + kvh) * (long long)(HSV * 16) + c) * BS + t % BS;
-        f32x4 vv[HSV];
-#pragma unroll
-        for (int dt = 0; dt < HSV; ++dt) vv[dt] = ld4(vr + (long long)dt * 16 * BS);
+        for (int e = 0; e < 4; ++e) a4[e] = __shfl(alpha, 4 * g + e, 64);
 #pragma unroll
         for (int dt = 0; dt < HSV; ++dt)
 #pragma unroll
-          for (int j = 0; j < 4; ++j) o[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(st[kt][j], vv[dt][j], o[dt], 0, 0, 0);
+          for (int e = 0; e < 4; ++e) o[dt][e] *= a4[e];
+#pragma unroll
+        for (int kt = 0; kt < 4; ++kt) {
+          // V^T of this lane's dimension 16 dt + c at keys t0 + 16 kt + 4 g .. + 3 (within one block)
+          const int t = min(t0 + 16 * kt + 4 * g, pos_max) & ~3;
+          const long long blk = table[t / BS];
+          const T* vr = vcache + ((blk * a.nkv + kvh) * (long long)(HSV * 16) + c) * BS + t % BS;
+          f32x4 vv[HSV];
+#pragma unroll
+          for (int dt = 0; dt < HSV; ++dt) vv[dt] = ld4(vr + (long long)dt * 16 * BS);
+#pragma unroll
+          for (int dt = 0; dt < HSV; ++dt)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) o[dt] = __builtin_amdgcn_mfma_f32_16x16x4f32(st[kt][j], vv[dt][j], o[dt], 0, 0, 0);
+        }
       }
       t0 += 64;
       if (t0 >= kept_end && t0 < wstart) t0 = wstart;  // from the kept first tokens on to the window
+    }
+  }
+  // the wavefronts' partial results meet: 1 .. SPLIT - 1 leave theirs in LDS, the first merges them in order
+  __syncthreads();  // (the queries are no longer needed: their room is taken)
+  if (wave > 0) {
+    float* part = smem + (wave - 1) * PART;
+#pragma unroll
+    for (int dt = 0; dt < HSV; ++dt) *(f32x4*)(part + (dt * 64 + lane) * 4) = o[dt];
+    if (g == 0) part[64 * HSV * 4 + c] = m, part[64 * HSV * 4 + 16 + c] = l;
+  }
+  __syncthreads();
+  if (wave > 0) return;
+  float m4[4];  // the running maximum of the rows 4 g + e that this lane's accumulators belong to
+#pragma unroll
+  for (int e = 0; e < 4; ++e) m4[e] = __shfl(m, 4 * g + e, 64);
+  for (int w = 1; w < SPLIT; ++w) {
+    const float* part = smem + (w - 1) * PART;
+    const float mw = part[64 * HSV * 4 + c], lw = part[64 * HSV * 4 + 16 + c];
+    const float m_new = fmaxf(m, mw);
+    const bool none = m_new == -INFINITY;
+    l = none ? 0.f : l * expf(m - m_new) + lw * expf(mw - m_new);
+    m = m_new;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float mo = part[64 * HSV * 4 + 4 * g + e];
+      const float mn = fmaxf(m4[e], mo);
+      const float fa = mn == -INFINITY ? 0.f : expf(m4[e] - mn), fb = mn == -INFINITY ? 0.f : expf(mo - mn);
+      m4[e] = mn;
+#pragma unroll
+      for (int dt = 0; dt < HSV; ++dt) o[dt][e] = o[dt][e] * fa + part[(dt * 64 + lane) * 4 + e] * fb;
     }
   }
   float inv4[4];
@@ -273,7 +335,7 @@ bool launch_tiles(const void* q, void* out, const void* gate, const void* kcache
   dim3 grid(lq_ceil_div(a.rows, b.rows_per_tile), a.nh);
 #define LQ_SINK(HSV)                                                                                                  \
   case HSV:                                                                                                           \
-    sink_tiles_kernel<T, HSV><<<grid, 64, 0, stream>>>((const T*)q, (T*)out, (const T*)gate, (const T*)kcache,        \
+    sink_tiles_kernel<T, HSV><<<grid, 64 * SPLIT, 0, stream>>>((const T*)q, (T*)out, (const T*)gate, (const T*)kcache,        \
                                                        (const T*)vcache, b);                                          \
     return true;
   switch (a.VD / 16) {

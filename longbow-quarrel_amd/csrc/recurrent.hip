@@ -123,35 +123,69 @@ __global__ __launch_bounds__(256) void conv_state_kernel(const float* __restrict
 
 // ---------------------------------------------------------------- the scans
 // A head's state is [columns P][state size N] in memory.  A thread owns, of one column, the entries n = i LN + l
-// (i = 0 .. slab - 1): LN threads share a column, LN a power of two, slab = ceil(N / LN) <= 16.  Sums over n are
-// a thread's own entries in ascending i, then an exchange over the LN lanes.
-constexpr int SLAB = 16;
-constexpr int SCAN_CHUNK = 8;  // tokens whose shared inputs are staged in LDS at a time
+// (i = 0 .. slab - 1): LN threads share a column, LN the power of two with slab = ceil(N / LN) <= 8 (16 for states
+// beyond 512), which depends on the model's sizes only.  Sums over n are a thread's own entries in ascending i, then
+// an exchange over the LN lanes.  What the columns of a workgroup share of a token (B and C or q and k, the
+// workgroup's slice of x or v, the token's decay and step) is staged in LDS for a chunk of tokens at a time, two
+// buffers taking turns: the next chunk's loads are in flight while this chunk is computed.
+constexpr int PRE = 16;        // registers a thread lends to a chunk's loads of the shared rows
+constexpr int MAX_CHUNK = 16;  // tokens a chunk at most
 
+template <int CTRL>
+__device__ inline float dpp_swap(float v) {
+  return __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, false));
+}
+
+// the sum over the LN lanes of a column; every lane gets it
 template <int LN>
 __device__ inline float group_sum(float v) {
-#pragma unroll
-  for (int off = 1; off < LN; off <<= 1) v += __shfl_xor(v, off, LQ_WAVE);
+  if (LN >= 2) v += dpp_swap<0xB1>(v);    // lanes 1 apart (quad_perm [1,0,3,2])
+  if (LN >= 4) v += dpp_swap<0x4E>(v);    // 2 apart (quad_perm [2,3,0,1])
+  if (LN >= 8) v += dpp_swap<0x141>(v);   // the other quad of eight lanes (row_half_mirror)
+  if (LN >= 16) v += dpp_swap<0x140>(v);  // the other half of sixteen (row_mirror)
+  if (LN >= 32) v += __shfl_xor(v, 16, LQ_WAVE);
+  if (LN >= 64) v += __shfl_xor(v, 32, LQ_WAVE);
   return v;
 }
 
-// Mamba-2: S <- exp(-exp(A_log) dt) S + dt B x^T,  y = S^T C + D x,  dt = softplus(raw + bias)
-template <int LN>
-__global__ void ssd_scan_kernel(const float* __restrict__ x, int ldx, const float* __restrict__ Bm, int ldb,
-                                const float* __restrict__ Cm, int ldc, const float* __restrict__ dt, int lddt,
-                                const float* __restrict__ dt_bias, const float* __restrict__ a_log,
-                                const float* __restrict__ d_skip, float* __restrict__ state, float* __restrict__ y,
-                                int ldy, int heads, int P, int N, int groups, const int* __restrict__ seq_slot,
-                                const int* __restrict__ cu_rows) {
-  extern __shared__ float lds[];  // [chunk][B: N | C: N] then [chunk][decay, dt]
-  const int b = blockIdx.x / heads, h = blockIdx.x % heads, g = h / (heads / groups);
-  const int cols = blockDim.x / LN;
-  const int l = threadIdx.x % LN, p = blockIdx.y * cols + threadIdx.x / LN;
+struct ScanShape {
+  int heads, groups, P, N;  // groups: of the shared rows (state-space groups, q/k heads)
+  const int *seq_slot, *cu_rows;
+};
+
+// The chunk-wise staging that both scans share.  `a`, `b`: the two shared rows of a token ([rows, groups * N] each),
+// `x`: the per-column input ([rows, heads * P]).  LDS of one buffer: [TT][2 N] then [TT][cols] then [TT][2].
+template <int LN, int SLAB>
+struct Stage {
+  static constexpr int PER = LN >= 32 ? LN / 16 : 1;  // entries of a token's two shared rows a thread (2 N <= 16 LN)
+  static constexpr int TT = PRE / PER / (SLAB / 8);   // tokens a chunk (fewer of the widest rows: LDS)
+  static constexpr int XPRE = TT / LN > 0 ? TT / LN : 1;  // chunk * cols / threads at most
+  float ab[PRE];
+  float xs[XPRE];
+  float s0, s1;
+};
+
+template <int LN, int SLAB>
+__global__ __launch_bounds__(256, 2) void ssd_scan_kernel(const float* __restrict__ x, int ldx,
+                                                       const float* __restrict__ Bm, int ldb,
+                                                       const float* __restrict__ Cm, int ldc,
+                                                       const float* __restrict__ dt, int lddt,
+                                                       const float* __restrict__ dt_bias,
+                                                       const float* __restrict__ a_log,
+                                                       const float* __restrict__ d_skip, float* __restrict__ state,
+                                                       float* __restrict__ y, int ldy, ScanShape sh) {
+  extern __shared__ float lds[];
+  const int heads = sh.heads, P = sh.P, N = sh.N;
+  constexpr int TT = Stage<LN, SLAB>::TT, PER = Stage<LN, SLAB>::PER;
+  const int b = blockIdx.x / heads, h = blockIdx.x % heads, g = h / (heads / sh.groups);
+  const int threads = blockDim.x, cols = threads / LN, tid = threadIdx.x;
+  const int l = tid % LN, col = tid / LN, p0 = blockIdx.y * cols, p = p0 + col;
   const bool live = p < P;
   const int slab = (N + LN - 1) / LN;
-  const long long r0 = cu_rows[b], r1 = cu_rows[b + 1];
-  float* sp = state + (((long long)seq_slot[b] * heads + h) * P + (live ? p : 0)) * N;
-  float* scal = lds + SCAN_CHUNK * 2 * N;
+  const long long r0 = sh.cu_rows[b], r1 = sh.cu_rows[b + 1];
+  float* sp = state + (((long long)sh.seq_slot[b] * heads + h) * P + (live ? p : 0)) * N;
+  constexpr int NP = LN * SLAB;  // a shared row in LDS, padded with zeros: entries past N take part as zeros
+  const int buf_floats = TT * (2 * NP + 2 * cols + 2);  // shared rows, inputs, decay and step, outputs
   float S[SLAB];
 #pragma unroll
   for (int i = 0; i < SLAB; ++i) {
@@ -159,38 +193,107 @@ __global__ void ssd_scan_kernel(const float* __restrict__ x, int ldx, const floa
     S[i] = (live && i < slab && n < N) ? sp[n] : 0.f;
   }
   const float A = -expf(a_log[h]), bias = dt_bias[h], D = d_skip[h];
-  for (long long c0 = r0; c0 < r1; c0 += SCAN_CHUNK) {
-    const int nt = (int)min((long long)SCAN_CHUNK, r1 - c0);
-    __syncthreads();  // the chunk before has been read
-    for (int e = threadIdx.x; e < nt * N; e += blockDim.x) {
-      const int t = e / N, n = e - t * N;
-      lds[t * 2 * N + n] = Bm[(c0 + t) * ldb + g * N + n];
-      lds[t * 2 * N + N + n] = Cm[(c0 + t) * ldc + g * N + n];
+  Stage<LN, SLAB> st;
+
+  auto fetch = [&](long long c0, int nt) {  // the chunk's loads, into registers
+#pragma unroll
+    for (int t = 0; t < TT; ++t)
+#pragma unroll
+      for (int jj = 0; jj < PER; ++jj) {
+        const int j = tid + jj * threads;
+        if (t < nt && j < 2 * N)
+          st.ab[t * PER + jj] = j < N ? Bm[(c0 + t) * ldb + g * N + j] : Cm[(c0 + t) * ldc + g * N + j - N];
+      }
+#pragma unroll
+    for (int i = 0; i < Stage<LN, SLAB>::XPRE; ++i) {
+      const int e = tid + i * threads;
+      if (e < nt * cols) {
+        const int t = e / cols, c = e - t * cols;
+        st.xs[i] = p0 + c < P ? x[(c0 + t) * ldx + h * P + p0 + c] : 0.f;
+      }
     }
-    if (threadIdx.x < nt) {
-      const float step = softplus_f(dt[(c0 + threadIdx.x) * lddt + h] + bias);
-      scal[2 * threadIdx.x] = expf(A * step);
-      scal[2 * threadIdx.x + 1] = step;
+    if (tid < nt) st.s0 = dt[(c0 + tid) * lddt + h];
+  };
+  auto stash = [&](float* buf, int nt) {  // registers to LDS
+#pragma unroll
+    for (int t = 0; t < TT; ++t)
+#pragma unroll
+      for (int jj = 0; jj < PER; ++jj) {
+        const int c = tid + jj * threads;
+        if (t < nt && c < 2 * N) buf[t * 2 * NP + (c < N ? c : NP + c - N)] = st.ab[t * PER + jj];
+      }
+#pragma unroll
+    for (int i = 0; i < Stage<LN, SLAB>::XPRE; ++i) {
+      const int e = tid + i * threads;
+      if (e < nt * cols) buf[TT * 2 * NP + e] = st.xs[i];
     }
-    __syncthreads();
-    for (int t = 0; t < nt; ++t) {
-      const float decay = scal[2 * t], step = scal[2 * t + 1];
-      const float xv = live ? x[(c0 + t) * ldx + h * P + p] : 0.f;
-      const float dx = step * xv;
-      const float* Bs = lds + t * 2 * N;
-      const float* Cs = Bs + N;
+    if (tid < nt) {
+      const float step = softplus_f(st.s0 + bias);
+      buf[TT * (2 * NP + cols) + 2 * tid] = expf(A * step);
+      buf[TT * (2 * NP + cols) + 2 * tid + 1] = step;
+    }
+  };
+
+  auto flush = [&](const float* buf, long long c0, int nt) {  // a chunk's outputs, from LDS to memory
+    for (int e = tid; e < nt * cols; e += threads) {
+      const int t = e / cols, c = e - t * cols;
+      if (p0 + c < P) y[(c0 + t) * ldy + h * P + p0 + c] = buf[TT * (2 * NP + cols + 2) + e];
+    }
+  };
+  for (int e = tid; e < 2 * buf_floats; e += threads) lds[e] = 0.f;
+  __syncthreads();
+  int cur = 0;
+  if (r1 > r0) {
+    const int nt = (int)min((long long)TT, r1 - r0);
+    fetch(r0, nt);
+    stash(lds, nt);
+  }
+  __syncthreads();
+  for (long long c0 = r0; c0 < r1; c0 += TT, cur ^= 1) {
+    const int nt = (int)min((long long)TT, r1 - c0);
+    const int next = (int)min((long long)TT, r1 - c0 - TT);
+    if (c0 > r0) flush(lds + (cur ^ 1) * buf_floats, c0 - TT, TT);  // the chunk before: its stores are long done
+    if (next > 0) fetch(c0 + TT, next);                             // when the wait for these loads comes
+    float* buf = lds + cur * buf_floats;
+    const float* scal = buf + TT * (2 * NP + cols);
+    float* outs = buf + TT * (2 * NP + cols + 2);
+    // a token's operands are read from LDS into registers while the token before it is computed (two sets of
+    // registers take turns: a read placed after the LDS store of a result could not pass it)
+    struct Tok {
+      float b[SLAB], c[SLAB], decay, step, x;
+    };
+    auto load = [&](Tok& k, int t) {
+      k.decay = scal[2 * t], k.step = scal[2 * t + 1], k.x = buf[TT * 2 * NP + t * cols + col];
+#pragma unroll
+      for (int i = 0; i < SLAB; ++i) k.b[i] = buf[t * 2 * NP + i * LN + l], k.c[i] = buf[t * 2 * NP + NP + i * LN + l];
+    };
+    auto compute = [&](const Tok& k, int t) {
+      const float dx = k.step * k.x;
       float acc = 0.f;
 #pragma unroll
       for (int i = 0; i < SLAB; ++i) {
-        const int n = i * LN + l;
-        if (i < slab && n < N) {
-          S[i] = fmaf(Bs[n], dx, decay * S[i]);
-          acc = fmaf(S[i], Cs[n], acc);
-        }
+        S[i] = fmaf(k.b[i], dx, k.decay * S[i]);
+        acc = fmaf(S[i], k.c[i], acc);
       }
       acc = group_sum<LN>(acc);
-      if (live && l == 0) y[(c0 + t) * ldy + h * P + p] = fmaf(D, xv, acc);
+      if (l == 0) outs[t * cols + col] = fmaf(D, k.x, acc);
+    };
+    Tok ka, kb;
+    load(ka, 0);
+    for (int t = 0; t < nt; t += 2) {
+      if (t + 1 < nt) load(kb, t + 1);
+      compute(ka, t);
+      if (t + 1 < nt) {
+        if (t + 2 < nt) load(ka, t + 2);
+        compute(kb, t + 1);
+      }
     }
+    if (next > 0) stash(lds + (cur ^ 1) * buf_floats, next);
+    __syncthreads();
+  }
+  if (r1 > r0) {  // the last chunk's outputs (cur has moved on once more)
+    const long long rows = r1 - r0, last = r0 + (rows - 1) / TT * TT;
+    flush(lds + (cur ^ 1) * buf_floats, last, (int)(r1 - last));
   }
   if (live) {
 #pragma unroll
@@ -203,83 +306,153 @@ __global__ void ssd_scan_kernel(const float* __restrict__ x, int ldx, const floa
 
 // Gated delta rule: S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q, with q and k made unit
 // vectors (x / sqrt(sum x^2 + unit_eps)), q times q_scale, beta = sigmoid(raw), g = exp(-exp(A_log) softplus(raw + bias)).
-template <int LN>
-__global__ void delta_scan_kernel(const float* __restrict__ q, int ldq, const float* __restrict__ k, int ldk,
-                                  const float* __restrict__ v, int ldv, const float* __restrict__ beta, int ldbeta,
-                                  const float* __restrict__ a, int lda, const float* __restrict__ dt_bias,
-                                  const float* __restrict__ a_log, float* __restrict__ state, float* __restrict__ out,
-                                  int ldo, int heads, int kv_heads, int Dk, int P, float q_scale, float unit_eps,
-                                  const int* __restrict__ seq_slot, const int* __restrict__ cu_rows) {
-  extern __shared__ float lds[];  // [chunk][q: Dk | k: Dk] then [chunk][decay, beta]
-  const int b = blockIdx.x / heads, h = blockIdx.x % heads, j = h / (heads / kv_heads);
-  const int cols = blockDim.x / LN;
-  const int l = threadIdx.x % LN, p = blockIdx.y * cols + threadIdx.x / LN;
+// (ScanShape: groups = q/k heads, N = key size.)
+template <int LN, int SLAB>
+__global__ __launch_bounds__(256, 2) void delta_scan_kernel(const float* __restrict__ q, int ldq,
+                                                         const float* __restrict__ k, int ldk,
+                                                         const float* __restrict__ v, int ldv,
+                                                         const float* __restrict__ beta, int ldbeta,
+                                                         const float* __restrict__ a, int lda,
+                                                         const float* __restrict__ dt_bias,
+                                                         const float* __restrict__ a_log, float* __restrict__ state,
+                                                         float* __restrict__ out, int ldo, float q_scale,
+                                                         float unit_eps, ScanShape sh) {
+  extern __shared__ float lds[];
+  const int heads = sh.heads, P = sh.P, N = sh.N;
+  constexpr int TT = Stage<LN, SLAB>::TT, PER = Stage<LN, SLAB>::PER;
+  const int b = blockIdx.x / heads, h = blockIdx.x % heads, j = h / (heads / sh.groups);
+  const int threads = blockDim.x, cols = threads / LN, tid = threadIdx.x;
+  const int l = tid % LN, col = tid / LN, p0 = blockIdx.y * cols, p = p0 + col;
   const bool live = p < P;
-  const int slab = (Dk + LN - 1) / LN;
-  const long long r0 = cu_rows[b], r1 = cu_rows[b + 1];
-  float* sp = state + (((long long)seq_slot[b] * heads + h) * P + (live ? p : 0)) * Dk;
-  float* scal = lds + SCAN_CHUNK * 2 * Dk;
+  const int slab = (N + LN - 1) / LN;
+  const long long r0 = sh.cu_rows[b], r1 = sh.cu_rows[b + 1];
+  float* sp = state + (((long long)sh.seq_slot[b] * heads + h) * P + (live ? p : 0)) * N;
+  constexpr int NP = LN * SLAB;  // a shared row in LDS, padded with zeros: entries past N take part as zeros
+  const int buf_floats = TT * (2 * NP + 2 * cols + 2);  // shared rows, inputs, decay and step, outputs
   float S[SLAB];
 #pragma unroll
   for (int i = 0; i < SLAB; ++i) {
     const int n = i * LN + l;
-    S[i] = (live && i < slab && n < Dk) ? sp[n] : 0.f;
+    S[i] = (live && i < slab && n < N) ? sp[n] : 0.f;
   }
   const float A = -expf(a_log[h]), bias = dt_bias[h];
-  for (long long c0 = r0; c0 < r1; c0 += SCAN_CHUNK) {
-    const int nt = (int)min((long long)SCAN_CHUNK, r1 - c0);
-    __syncthreads();
-    for (int e = threadIdx.x; e < nt * Dk; e += blockDim.x) {
-      const int t = e / Dk, n = e - t * Dk;
-      lds[t * 2 * Dk + n] = q[(c0 + t) * ldq + j * Dk + n];
-      lds[t * 2 * Dk + Dk + n] = k[(c0 + t) * ldk + j * Dk + n];
+  Stage<LN, SLAB> st;
+
+  auto fetch = [&](long long c0, int nt) {
+#pragma unroll
+    for (int t = 0; t < TT; ++t)
+#pragma unroll
+      for (int jj = 0; jj < PER; ++jj) {
+        const int c = tid + jj * threads;
+        if (t < nt && c < 2 * N)
+          st.ab[t * PER + jj] = c < N ? q[(c0 + t) * ldq + j * N + c] : k[(c0 + t) * ldk + j * N + c - N];
+      }
+#pragma unroll
+    for (int i = 0; i < Stage<LN, SLAB>::XPRE; ++i) {
+      const int e = tid + i * threads;
+      if (e < nt * cols) {
+        const int t = e / cols, c = e - t * cols;
+        st.xs[i] = p0 + c < P ? v[(c0 + t) * ldv + h * P + p0 + c] : 0.f;
+      }
     }
-    if (threadIdx.x < nt) {
-      scal[2 * threadIdx.x] = expf(A * softplus_f(a[(c0 + threadIdx.x) * lda + h] + bias));
-      scal[2 * threadIdx.x + 1] = sigmoid_f(beta[(c0 + threadIdx.x) * ldbeta + h]);
+    if (tid < nt) {
+      st.s0 = a[(c0 + tid) * lda + h];
+      st.s1 = beta[(c0 + tid) * ldbeta + h];
     }
-    __syncthreads();
-    for (int t = 0; t < nt; ++t) {
-      const float decay = scal[2 * t], bt = scal[2 * t + 1];
-      const float vv = live ? v[(c0 + t) * ldv + h * P + p] : 0.f;
-      const float* Qs = lds + t * 2 * Dk;
-      const float* Ks = Qs + Dk;
-      float kk[SLAB], qq[SLAB];
-      float ssq = 0.f, ssk = 0.f;
+  };
+  auto stash = [&](float* buf, int nt) {
+#pragma unroll
+    for (int t = 0; t < TT; ++t)
+#pragma unroll
+      for (int jj = 0; jj < PER; ++jj) {
+        const int c = tid + jj * threads;
+        if (t < nt && c < 2 * N) buf[t * 2 * NP + (c < N ? c : NP + c - N)] = st.ab[t * PER + jj];
+      }
+#pragma unroll
+    for (int i = 0; i < Stage<LN, SLAB>::XPRE; ++i) {
+      const int e = tid + i * threads;
+      if (e < nt * cols) buf[TT * 2 * NP + e] = st.xs[i];
+    }
+    if (tid < nt) {
+      buf[TT * (2 * NP + cols) + 2 * tid] = expf(A * softplus_f(st.s0 + bias));
+      buf[TT * (2 * NP + cols) + 2 * tid + 1] = sigmoid_f(st.s1);
+    }
+  };
+
+  auto flush = [&](const float* buf, long long c0, int nt) {  // a chunk's outputs, from LDS to memory
+    for (int e = tid; e < nt * cols; e += threads) {
+      const int t = e / cols, c = e - t * cols;
+      if (p0 + c < P) out[(c0 + t) * ldo + h * P + p0 + c] = buf[TT * (2 * NP + cols + 2) + e];
+    }
+  };
+  for (int e = tid; e < 2 * buf_floats; e += threads) lds[e] = 0.f;
+  __syncthreads();
+  int cur = 0;
+  if (r1 > r0) {
+    const int nt = (int)min((long long)TT, r1 - r0);
+    fetch(r0, nt);
+    stash(lds, nt);
+  }
+  __syncthreads();
+  for (long long c0 = r0; c0 < r1; c0 += TT, cur ^= 1) {
+    const int nt = (int)min((long long)TT, r1 - c0);
+    const int next = (int)min((long long)TT, r1 - c0 - TT);
+    if (c0 > r0) flush(lds + (cur ^ 1) * buf_floats, c0 - TT, TT);  // the chunk before: its stores are long done
+    if (next > 0) fetch(c0 + TT, next);                             // when the wait for these loads comes
+    float* buf = lds + cur * buf_floats;
+    const float* scal = buf + TT * (2 * NP + cols);
+    float* outs = buf + TT * (2 * NP + cols + 2);
+    struct Tok {  // (as in the state-space scan: the next token's operands are read while this one is computed)
+      float q[SLAB], k[SLAB], decay, beta, v;
+    };
+    auto load = [&](Tok& k, int t) {
+      k.decay = scal[2 * t], k.beta = scal[2 * t + 1], k.v = buf[TT * 2 * NP + t * cols + col];
+#pragma unroll
+      for (int i = 0; i < SLAB; ++i) k.q[i] = buf[t * 2 * NP + i * LN + l], k.k[i] = buf[t * 2 * NP + NP + i * LN + l];
+    };
+    auto compute = [&](const Tok& k, int t) {
+      float ssq = 0.f, ssk = 0.f, sk = 0.f;
 #pragma unroll
       for (int i = 0; i < SLAB; ++i) {
-        const int n = i * LN + l;
-        const bool in = i < slab && n < Dk;
-        kk[i] = in ? Ks[n] : 0.f;
-        qq[i] = in ? Qs[n] : 0.f;
-        ssk = fmaf(kk[i], kk[i], ssk);
-        ssq = fmaf(qq[i], qq[i], ssq);
+        ssk = fmaf(k.k[i], k.k[i], ssk);
+        ssq = fmaf(k.q[i], k.q[i], ssq);
+        S[i] *= k.decay;
+        sk = fmaf(S[i], k.k[i], sk);  // with k as it came: the unit norm is one factor of the sum
       }
       const float kinv = 1.f / sqrtf(group_sum<LN>(ssk) + unit_eps);
       const float qinv = q_scale / sqrtf(group_sum<LN>(ssq) + unit_eps);
-      float sk = 0.f;
-#pragma unroll
-      for (int i = 0; i < SLAB; ++i) {
-        kk[i] *= kinv;
-        S[i] *= decay;
-        sk = fmaf(S[i], kk[i], sk);
-      }
-      const float u = bt * (vv - group_sum<LN>(sk));
+      const float uk = k.beta * (k.v - group_sum<LN>(sk) * kinv) * kinv;
       float o = 0.f;
 #pragma unroll
       for (int i = 0; i < SLAB; ++i) {
-        S[i] = fmaf(kk[i], u, S[i]);
-        o = fmaf(S[i], qq[i], o);
+        S[i] = fmaf(k.k[i], uk, S[i]);
+        o = fmaf(S[i], k.q[i], o);
       }
       o = group_sum<LN>(o) * qinv;
-      if (live && l == 0) out[(c0 + t) * ldo + h * P + p] = o;
+      if (l == 0) outs[t * cols + col] = o;
+    };
+    Tok ka, kb;
+    load(ka, 0);
+    for (int t = 0; t < nt; t += 2) {
+      if (t + 1 < nt) load(kb, t + 1);
+      compute(ka, t);
+      if (t + 1 < nt) {
+        if (t + 2 < nt) load(ka, t + 2);
+        compute(kb, t + 1);
+      }
     }
+    if (next > 0) stash(lds + (cur ^ 1) * buf_floats, next);
+    __syncthreads();
+  }
+  if (r1 > r0) {  // the last chunk's outputs (cur has moved on once more)
+    const long long rows = r1 - r0, last = r0 + (rows - 1) / TT * TT;
+    flush(lds + (cur ^ 1) * buf_floats, last, (int)(r1 - last));
   }
   if (live) {
 #pragma unroll
     for (int i = 0; i < SLAB; ++i) {
       const int n = i * LN + l;
-      if (i < slab && n < Dk) sp[n] = S[i];
+      if (i < slab && n < N) sp[n] = S[i];
     }
   }
 }
@@ -332,18 +505,25 @@ __global__ void rmsnorm_mean_kernel(MeanInputs in, int n_in, float eps, float* _
   }
 }
 
-int scan_lanes(int n) {  // the power of two LN with ceil(n / LN) <= SLAB
-  int ln = 1;
-  while ((n + ln - 1) / ln > SLAB) ln <<= 1;
-  return ln;
-}
+// How a scan over states of N entries a column and P columns a head is launched; all of it follows from the
+// model's sizes, nothing from the step, so that a token's sums are the same in every launch.
+struct ScanLaunch {
+  int ln, slab, threads, cols, tt;
+  size_t lds;
+};
 
-// threads a workgroup: as many columns as fit, fewer where the launch would otherwise leave compute units idle
-int scan_threads(int ln, int P, long long seq_heads) {
-  int threads = 256;
-  while (threads > 64 && (threads / ln >= 2 * P || seq_heads * lq_ceil_div(P, threads / ln) < 2ll * lq_compute_units()))
-    threads >>= 1;
-  return threads < ln ? ln : threads;
+bool scan_launch(int N, int P, ScanLaunch& s) {
+  s.slab = N > 512 ? 16 : 8;
+  s.ln = 1;
+  while ((N + s.ln - 1) / s.ln > s.slab) s.ln <<= 1;
+  if (s.ln > 64) return false;
+  const int per = s.ln >= 32 ? s.ln / 16 : 1;  // as Stage<LN, SLAB> has them
+  s.tt = PRE / per / (s.slab / 8);
+  s.threads = (P * s.ln + 63) / 64 * 64;
+  if (s.threads > 256 || 2 * N > per * s.threads) s.threads = 256;  // (2 N <= 16 LN <= per * 256)
+  s.cols = s.threads / s.ln;
+  s.lds = 2 * (size_t)s.tt * (2 * s.ln * s.slab + 2 * s.cols + 2) * sizeof(float);  // (rows padded to LN * slab)
+  return s.lds <= 64 * 1024;
 }
 
 }  // namespace
@@ -424,15 +604,16 @@ extern "C" int lq_causal_conv(const float* x, int ldx, const float* w, const flo
   return 0;
 }
 
-#define LQ_SCAN_LANES(LAUNCH)          \
-  switch (ln) {                        \
-    case 1: LAUNCH(1); break;          \
-    case 2: LAUNCH(2); break;          \
-    case 4: LAUNCH(4); break;          \
-    case 8: LAUNCH(8); break;          \
-    case 16: LAUNCH(16); break;        \
-    case 32: LAUNCH(32); break;        \
-    default: LAUNCH(64); break;        \
+#define LQ_SCAN_LANES(LAUNCH)                \
+  switch (cfg.slab == 16 ? 128 : cfg.ln) {   \
+    case 1: LAUNCH(1, 8); break;             \
+    case 2: LAUNCH(2, 8); break;             \
+    case 4: LAUNCH(4, 8); break;             \
+    case 8: LAUNCH(8, 8); break;             \
+    case 16: LAUNCH(16, 8); break;           \
+    case 32: LAUNCH(32, 8); break;           \
+    case 64: LAUNCH(64, 8); break;           \
+    default: LAUNCH(64, 16); break;          \
   }
 
 // x [rows, heads * P], B and C [rows, groups * N], dt [rows, heads] (before its softplus), state
@@ -442,18 +623,16 @@ extern "C" int lq_ssd_scan(const float* x, int ldx, const float* Bm, int ldb, co
                            int ldy, int heads, int P, int N, int groups, const int* seq_slot, const int* cu_rows, int batch,
                            hipStream_t stream) {
   LQ_REQUIRE(heads > 0 && P > 0 && N > 0 && groups > 0 && heads % groups == 0 && batch > 0, "ssd_scan: bad sizes");
-  LQ_REQUIRE(N <= SLAB * 64, "ssd_scan: state size %d exceeds %d", N, SLAB * 64);
   LQ_REQUIRE(ldx >= heads * P && ldy >= heads * P && ldb >= groups * N && ldc >= groups * N && lddt >= heads,
              "ssd_scan: a row stride is smaller than its row");
   LQ_REQUIRE(x && Bm && Cm && dt && dt_bias && a_log && d_skip && state && y && seq_slot && cu_rows, "ssd_scan: null pointer");
-  const int ln = scan_lanes(N);
-  const int threads = scan_threads(ln, P, (long long)batch * heads);
-  dim3 grid((unsigned)(batch * heads), lq_ceil_div(P, threads / ln));
-  const size_t lds = (size_t)SCAN_CHUNK * (2 * N + 2) * sizeof(float);
-  LQ_REQUIRE(lds <= 64 * 1024, "ssd_scan: state size %d needs too much LDS", N);
-#define LQ_SSD(LN)                                                                                                      \
-  ssd_scan_kernel<LN><<<grid, threads, lds, stream>>>(x, ldx, Bm, ldb, Cm, ldc, dt, lddt, dt_bias, a_log, d_skip, state, \
-                                                      y, ldy, heads, P, N, groups, seq_slot, cu_rows)
+  ScanLaunch cfg;
+  LQ_REQUIRE(scan_launch(N, P, cfg), "ssd_scan: state size %d is too large", N);
+  dim3 grid((unsigned)(batch * heads), lq_ceil_div(P, cfg.cols));
+  ScanShape sh = {heads, groups, P, N, seq_slot, cu_rows};
+#define LQ_SSD(LN, SL)                                                                                              \
+  ssd_scan_kernel<LN, SL><<<grid, cfg.threads, cfg.lds, stream>>>(x, ldx, Bm, ldb, Cm, ldc, dt, lddt, dt_bias, a_log, \
+                                                                  d_skip, state, y, ldy, sh)
   LQ_SCAN_LANES(LQ_SSD)
 #undef LQ_SSD
   LQ_CHECK_LAUNCH("ssd_scan");
@@ -467,19 +646,16 @@ extern "C" int lq_delta_scan(const float* q, int ldq, const float* k, int ldk, c
                              float* out, int ldo, int heads, int kv_heads, int Dk, int P, float q_scale, float unit_eps,
                              const int* seq_slot, const int* cu_rows, int batch, hipStream_t stream) {
   LQ_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && Dk > 0 && P > 0 && batch > 0, "delta_scan: bad sizes");
-  LQ_REQUIRE(Dk <= SLAB * 64, "delta_scan: key size %d exceeds %d", Dk, SLAB * 64);
   LQ_REQUIRE(ldq >= kv_heads * Dk && ldk >= kv_heads * Dk && ldv >= heads * P && ldo >= heads * P && ldbeta >= heads &&
                  lda >= heads, "delta_scan: a row stride is smaller than its row");
   LQ_REQUIRE(q && k && v && beta && a && dt_bias && a_log && state && out && seq_slot && cu_rows, "delta_scan: null pointer");
-  const int ln = scan_lanes(Dk);
-  const int threads = scan_threads(ln, P, (long long)batch * heads);
-  dim3 grid((unsigned)(batch * heads), lq_ceil_div(P, threads / ln));
-  const size_t lds = (size_t)SCAN_CHUNK * (2 * Dk + 2) * sizeof(float);
-  LQ_REQUIRE(lds <= 64 * 1024, "delta_scan: key size %d needs too much LDS", Dk);
-#define LQ_DELTA(LN)                                                                                                 \
-  delta_scan_kernel<LN><<<grid, threads, lds, stream>>>(q, ldq, k, ldk, v, ldv, beta, ldbeta, a, lda, dt_bias, a_log,  \
-                                                        state, out, ldo, heads, kv_heads, Dk, P, q_scale, unit_eps,    \
-                                                        seq_slot, cu_rows)
+  ScanLaunch cfg;
+  LQ_REQUIRE(scan_launch(Dk, P, cfg), "delta_scan: key size %d is too large", Dk);
+  dim3 grid((unsigned)(batch * heads), lq_ceil_div(P, cfg.cols));
+  ScanShape sh = {heads, kv_heads, P, Dk, seq_slot, cu_rows};
+#define LQ_DELTA(LN, SL)                                                                                             \
+  delta_scan_kernel<LN, SL><<<grid, cfg.threads, cfg.lds, stream>>>(q, ldq, k, ldk, v, ldv, beta, ldbeta, a, lda,      \
+                                                                    dt_bias, a_log, state, out, ldo, q_scale, unit_eps, sh)
   LQ_SCAN_LANES(LQ_DELTA)
 #undef LQ_DELTA
   LQ_CHECK_LAUNCH("delta_scan");
