@@ -486,21 +486,28 @@ struct MeanInputs {
   const float* w[4];
 };
 
-// out = (1 / n) sum_i x_i / rms(x_i) w_i, row by row
+// out = (1 / n) sum_i x_i / rms(x_i) w_i, row by row.  The branches' sums of squares are taken in one pass (their
+// loads are in flight together), each with the block's fixed tree.
 __global__ void rmsnorm_mean_kernel(MeanInputs in, int n_in, float eps, float* __restrict__ out, int width) {
   __shared__ float red[16];
   const long long r = blockIdx.x;
-  float inv[4];
-  for (int i = 0; i < n_in; ++i) {
-    const float* xr = in.x[i] + r * width;
-    float ss = 0.f;
-    for (int c = threadIdx.x; c < width; c += blockDim.x) ss = fmaf(xr[c], xr[c], ss);
-    inv[i] = 1.f / sqrtf(block_sum(ss, red) / width + eps);
+  float ss[4] = {0.f, 0.f, 0.f, 0.f};
+  for (int c = threadIdx.x; c < width; c += blockDim.x) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float v = i < n_in ? in.x[i][r * width + c] : 0.f;
+      ss[i] = fmaf(v, v, ss[i]);
+    }
   }
+  float inv[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) inv[i] = i < n_in ? 1.f / sqrtf(block_sum(ss[i], red) / width + eps) : 0.f;
   const float share = 1.f / n_in;
   for (int c = threadIdx.x; c < width; c += blockDim.x) {
     float acc = 0.f;
-    for (int i = 0; i < n_in; ++i) acc += in.x[i][r * width + c] * inv[i] * in.w[i][c];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (i < n_in) acc += in.x[i][r * width + c] * inv[i] * in.w[i][c];
     out[r * width + c] = acc * share;
   }
 }
@@ -698,7 +705,7 @@ extern "C" int lq_rmsnorm_mean(const float* stack, int n_in, const float* w0, co
     LQ_REQUIRE(i >= n_in || ws[i] != nullptr, "rmsnorm_mean: branch %d has no weight", i);
   }
   LQ_REQUIRE(stack && out, "rmsnorm_mean: null pointer");
-  rmsnorm_mean_kernel<<<rows, width >= 1024 ? 256 : 64, 0, stream>>>(in, n_in, eps, out, width);
+  rmsnorm_mean_kernel<<<rows, width >= 4096 ? 1024 : width >= 1024 ? 256 : 64, 0, stream>>>(in, n_in, eps, out, width);
   LQ_CHECK_LAUNCH("rmsnorm_mean");
   return 0;
 }
