@@ -157,8 +157,9 @@ struct ScanShape {
 // `x`: the per-column input ([rows, heads * P]).  LDS of one buffer: [TT][2 N] then [TT][cols] then [TT][2].
 template <int LN, int SLAB>
 struct Stage {
-  static constexpr int PER = LN >= 32 ? LN / 16 : 1;  // entries of a token's two shared rows a thread (2 N <= 16 LN)
-  static constexpr int TT = PRE / PER / (SLAB / 8);   // tokens a chunk (fewer of the widest rows: LDS)
+  // entries of a token's two shared rows a thread of 256 (2 N <= 2 SLAB LN)
+  static constexpr int PER = 2 * SLAB * LN > 256 ? 2 * SLAB * LN / 256 : 1;
+  static constexpr int TT = PRE / PER;  // tokens a chunk
   static constexpr int XPRE = TT / LN > 0 ? TT / LN : 1;  // chunk * cols / threads at most
   float ab[PRE];
   float xs[XPRE];
@@ -524,10 +525,10 @@ bool scan_launch(int N, int P, ScanLaunch& s) {
   s.ln = 1;
   while ((N + s.ln - 1) / s.ln > s.slab) s.ln <<= 1;
   if (s.ln > 64) return false;
-  const int per = s.ln >= 32 ? s.ln / 16 : 1;  // as Stage<LN, SLAB> has them
-  s.tt = PRE / per / (s.slab / 8);
+  const int per = 2 * s.slab * s.ln > 256 ? 2 * s.slab * s.ln / 256 : 1;  // as Stage<LN, SLAB> has them
+  s.tt = PRE / per;
   s.threads = (P * s.ln + 63) / 64 * 64;
-  if (s.threads > 256 || 2 * N > per * s.threads) s.threads = 256;  // (2 N <= 16 LN <= per * 256)
+  if (s.threads > 256 || 2 * N > per * s.threads) s.threads = 256;  // (2 N <= 2 slab LN <= per * 256)
   s.cols = s.threads / s.ln;
   s.lds = 2 * (size_t)s.tt * (2 * s.ln * s.slab + 2 * s.cols + 2) * sizeof(float);  // (rows padded to LN * slab)
   return s.lds <= 64 * 1024;

@@ -103,7 +103,7 @@ def test_a_window_that_keeps_first_tokens_gives_the_blocks_between_back():
     assert kept.blocks.taken_count == 0 and cm.free_blocks() == 6
 
 
-@pytest.mark.parametrize("name", ["a", "b", "c"])
+@pytest.mark.parametrize("name", ["a", "b", "c", "d"])
 def test_whole_prompts_and_token_by_token(cases, name):
     vc.whole_and_token_by_token(cases(name), TOL, lengths=(1, 2, 3, 70))
 

@@ -144,7 +144,8 @@ def test_short_convolution_carries_its_last_inputs(kn, taps, bias):
     assert at == lengths
 
 
-@pytest.mark.parametrize("sizes", [(4, 16, 24, 1), (3, 24, 20, 3), (2, 64, 130, 2), (6, 40, 64, 2), (1, 8, 300, 1)])
+@pytest.mark.parametrize("sizes", [(4, 16, 24, 1), (3, 24, 20, 3), (2, 64, 130, 2), (6, 40, 64, 2), (1, 8, 300, 1), (2, 12, 9, 2),
+                                   (1, 4, 600, 1)])
 def test_state_space_scan_in_portions(kn, sizes):
     H, P, N, G = sizes
     T = 45
@@ -174,7 +175,8 @@ def test_state_space_scan_in_portions(kn, sizes):
     assert torch.equal(y2[10:], torch.cat(got))
 
 
-@pytest.mark.parametrize("sizes", [(4, 2, 16, 32), (2, 2, 48, 16), (2, 1, 24, 40), (3, 3, 128, 64), (1, 1, 272, 8)])
+@pytest.mark.parametrize("sizes", [(4, 2, 16, 32), (2, 2, 48, 16), (2, 1, 24, 40), (3, 3, 128, 64), (1, 1, 272, 8), (3, 3, 12, 20),
+                                   (1, 1, 520, 4)])
 def test_gated_delta_rule_scan_in_portions(kn, sizes):
     H, G, D, P = sizes
     T = 40
@@ -265,7 +267,7 @@ def tol(dtype):
     return TOL_F32 if dtype == "float32" else TOL_BF16
 
 
-PARAMS = [(n, d) for n in ("a", "b", "c") for d in ("float32", "bfloat16")]
+PARAMS = [(n, d) for n in ("a", "b", "c", "d") for d in ("float32", "bfloat16")]
 
 
 @pytest.mark.parametrize("name,dtype", PARAMS)

@@ -60,7 +60,14 @@ CFG_C = _config(97, 64, 1.5, 1e-5, 0.25, [
     _parallel({"dim": 48, "vdim": 48, "heads": 1, "kv_heads": 1, "mask": {"size": 1, "keep_first": 1}, "scale": 1.0},
               {"conv": 1, "groups": 1, "heads": 1, "norm_groups": 8, "state": 16, "vdim": 64}, 32),
 ])
-CONFIGS = {"a": CFG_A, "b": CFG_B, "c": CFG_C}
+# D: nothing is a multiple of 8 (every product and every kernel takes its size-agnostic way), five taps, three
+# norm groups of 20, a state of 9
+CFG_D = _config(77, 100, 1.0, 1e-4, 0.8, [
+    _parallel({"dim": 20, "vdim": 12, "heads": 5, "kv_heads": 5, "mask": {"size": 3, "keep_first": 5}, "scale": 0.4},
+              {"conv": 5, "groups": 5, "heads": 5, "norm_groups": 3, "state": 9, "vdim": 12}, 50),
+    _delta({"conv": 2, "dim": 12, "heads": 3, "kv_heads": 3, "vdim": 20}, 52),
+])
+CONFIGS = {"a": CFG_A, "b": CFG_B, "c": CFG_C, "d": CFG_D}
 
 
 def make_weights(cfg: dict, seed: int, sharp: float = 1.0) -> Dict[str, torch.Tensor]:
