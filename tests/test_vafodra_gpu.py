@@ -145,7 +145,7 @@ def test_short_convolution_carries_its_last_inputs(kn, taps, bias):
 
 
 @pytest.mark.parametrize("sizes", [(4, 16, 24, 1), (3, 24, 20, 3), (2, 64, 130, 2), (6, 40, 64, 2), (1, 8, 300, 1), (2, 12, 9, 2),
-                                   (1, 4, 600, 1)])
+                                   (1, 4, 600, 1), (8, 64, 128, 2)])
 def test_state_space_scan_in_portions(kn, sizes):
     H, P, N, G = sizes
     T = 45
@@ -288,6 +288,15 @@ def test_unequal_batches_against_each_request_alone(cases, name, dtype):
 @pytest.mark.parametrize("name,dtype", PARAMS)
 def test_slots_and_blocks_that_are_used_again(cases, name, dtype):
     vc.slots_and_blocks_used_again(cases(name, dtype), tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sizes_of_a_small_real_model(cases, dtype):
+    case = cases("e", dtype)
+    t = vc.tokens(330, case.vocab, 6)
+    for cuts in ([330], [290], [130, 70, 100]):
+        assert vc.err(case.run_cut(t, cuts), case.want(t)) < tol(dtype), cuts
+    case.assert_idle()
 
 
 @pytest.mark.parametrize("name", ["a", "c"])

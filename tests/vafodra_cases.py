@@ -67,7 +67,15 @@ CFG_D = _config(77, 100, 1.0, 1e-4, 0.8, [
               {"conv": 5, "groups": 5, "heads": 5, "norm_groups": 3, "state": 9, "vdim": 12}, 50),
     _delta({"conv": 2, "dim": 12, "heads": 3, "kv_heads": 3, "vdim": 20}, 52),
 ])
-CONFIGS = {"a": CFG_A, "b": CFG_B, "c": CFG_C, "d": CFG_D}
+# E: head sizes, state and width of the kind that the fast kernels are made for
+CFG_E = _config(1000, 512, 1.0, 1e-5, 0.5, [
+    _parallel({"dim": 128, "vdim": 128, "heads": 4, "kv_heads": 1, "mask": {"size": 100, "keep_first": 3}, "scale": 0.09},
+              {"conv": 4, "groups": 2, "heads": 8, "norm_groups": 2, "state": 128, "vdim": 64}, 1792),
+    _delta({"conv": 4, "dim": 128, "heads": 4, "kv_heads": 2, "vdim": 128}, 1792),
+    _parallel({"dim": 64, "vdim": 256, "heads": 2, "kv_heads": 2, "mask": {"size": 200, "keep_first": 0}, "scale": 0.125},
+              {"conv": 4, "groups": 1, "heads": 16, "norm_groups": 1, "state": 64, "vdim": 32}, None),
+])
+CONFIGS = {"a": CFG_A, "b": CFG_B, "c": CFG_C, "d": CFG_D, "e": CFG_E}
 
 
 def make_weights(cfg: dict, seed: int, sharp: float = 1.0) -> Dict[str, torch.Tensor]:
