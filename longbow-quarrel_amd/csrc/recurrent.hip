@@ -148,6 +148,19 @@ __device__ inline float group_sum(float v) {
   return v;
 }
 
+// A launch of the state-space scan in segments, for few long sequences that would leave most of the chip idle: a
+// sequence of SEG_MIN_ROWS rows or more is cut into `nseg` segments (whole chunks), one workgroup each.  Pass 1: segment
+// 0 runs from the sequence's state, the others from zero without results, each leaving its end state and the product
+// of its decays; a short kernel chains them (S_end = prod(decay) S_start + S_end_from_zero); pass 2: segments 1 ..
+// run again from their true starts.  Twice the arithmetic, the segments side by side.  Shorter sequences of the same
+// launch run whole in pass 1.
+constexpr int SEG_MIN_ROWS = 512;
+constexpr int SEG_COUNT = 8;
+struct SegArgs {
+  int nseg, pass;  // nseg 1: no segments (pass 1 alone)
+  float *state, *decay;  // [sequences * heads][nseg][P][N], [sequences * heads][nseg]
+};
+
 struct ScanShape {
   int heads, groups, P, N;  // groups: of the shared rows (state-space groups, q/k heads)
   const int *seq_slot, *cu_rows;
@@ -174,7 +187,7 @@ __global__ __launch_bounds__(256, 2) void ssd_scan_kernel(const float* __restric
                                                        const float* __restrict__ dt_bias,
                                                        const float* __restrict__ a_log,
                                                        const float* __restrict__ d_skip, float* __restrict__ state,
-                                                       float* __restrict__ y, int ldy, ScanShape sh) {
+                                                       float* __restrict__ y, int ldy, ScanShape sh, SegArgs sg) {
   extern __shared__ float lds[];
   const int heads = sh.heads, P = sh.P, N = sh.N;
   constexpr int TT = Stage<LN, SLAB>::TT, PER = Stage<LN, SLAB>::PER;
@@ -183,15 +196,31 @@ __global__ __launch_bounds__(256, 2) void ssd_scan_kernel(const float* __restric
   const int l = tid % LN, col = tid / LN, p0 = blockIdx.y * cols, p = p0 + col;
   const bool live = p < P;
   const int slab = (N + LN - 1) / LN;
-  const long long r0 = sh.cu_rows[b], r1 = sh.cu_rows[b + 1];
+  long long r0 = sh.cu_rows[b], r1 = sh.cu_rows[b + 1];
+  // A long sequence of a launch in segments (see SegArgs): this workgroup's segment, where it starts from and
+  // where it leaves its state.
+  const int seg = blockIdx.z;
+  const int nseg = (sg.nseg > 1 && r1 - r0 >= SEG_MIN_ROWS) ? sg.nseg : 1;
+  if (seg >= nseg || (sg.pass == 2 && seg == 0)) return;
+  if (nseg > 1) {
+    const long long len = ((r1 - r0 + nseg - 1) / nseg + TT - 1) / TT * TT;
+    r0 = min(r1, r0 + seg * len);
+    r1 = min(r1, r0 + len);
+  }
+  const bool write_y = sg.pass == 2 || seg == 0;
   float* sp = state + (((long long)sh.seq_slot[b] * heads + h) * P + (live ? p : 0)) * N;
+  float* seg_sp = nseg > 1 ? sg.state + ((((long long)blockIdx.x * sg.nseg + seg) * P + (live ? p : 0)) * N) : nullptr;
+  const float* from = nseg > 1 && sg.pass == 2 ? seg_sp : sp;
+  const bool from_zero = nseg > 1 && sg.pass == 1 && seg > 0;
+  float* to = nseg == 1 ? sp : sg.pass == 1 ? seg_sp : nullptr;
+  float dprod = 1.f;  // the product of the segment's decays
   constexpr int NP = LN * SLAB;  // a shared row in LDS, padded with zeros: entries past N take part as zeros
   const int buf_floats = TT * (2 * NP + 2 * cols + 2);  // shared rows, inputs, decay and step, outputs
   float S[SLAB];
 #pragma unroll
   for (int i = 0; i < SLAB; ++i) {
     const int n = i * LN + l;
-    S[i] = (live && i < slab && n < N) ? sp[n] : 0.f;
+    S[i] = (live && !from_zero && i < slab && n < N) ? from[n] : 0.f;
   }
   const float A = -expf(a_log[h]), bias = dt_bias[h], D = d_skip[h];
   Stage<LN, SLAB> st;
@@ -236,6 +265,7 @@ __global__ __launch_bounds__(256, 2) void ssd_scan_kernel(const float* __restric
   };
 
   auto flush = [&](const float* buf, long long c0, int nt) {  // a chunk's outputs, from LDS to memory
+    if (!write_y) return;
     for (int e = tid; e < nt * cols; e += threads) {
       const int t = e / cols, c = e - t * cols;
       if (p0 + c < P) y[(c0 + t) * ldy + h * P + p0 + c] = buf[TT * (2 * NP + cols + 2) + e];
@@ -270,6 +300,7 @@ __global__ __launch_bounds__(256, 2) void ssd_scan_kernel(const float* __restric
     };
     auto compute = [&](const Tok& k, int t) {
       const float dx = k.step * k.x;
+      dprod *= k.decay;
       float acc = 0.f;
 #pragma unroll
       for (int i = 0; i < SLAB; ++i) {
@@ -296,14 +327,36 @@ __global__ __launch_bounds__(256, 2) void ssd_scan_kernel(const float* __restric
     const long long rows = r1 - r0, last = r0 + (rows - 1) / TT * TT;
     flush(lds + (cur ^ 1) * buf_floats, last, (int)(r1 - last));
   }
-  if (live) {
+  if (live && to != nullptr) {
 #pragma unroll
     for (int i = 0; i < SLAB; ++i) {
       const int n = i * LN + l;
-      if (i < slab && n < N) sp[n] = S[i];
+      if (i < slab && n < N) to[n] = S[i];
     }
   }
+  if (nseg > 1 && sg.pass == 1 && tid == 0 && blockIdx.y == 0) sg.decay[(long long)blockIdx.x * sg.nseg + seg] = dprod;
 }
+
+// Between the two passes of a launch in segments: segment 0 left the state at its true end, every other segment the
+// state it reaches from zero and the product of its decays.  In order, every segment's true start takes the place
+// of what it left, and the last segment's true end goes into the cache.
+__global__ __launch_bounds__(256) void ssd_chain_kernel(float* __restrict__ state, int heads, int PN, SegArgs sg,
+                                                        const int* __restrict__ seq_slot,
+                                                        const int* __restrict__ cu_rows) {
+  const int bh = blockIdx.x, b = bh / heads, h = bh % heads;
+  if (cu_rows[b + 1] - cu_rows[b] < SEG_MIN_ROWS) return;
+  const int e = blockIdx.y * 256 + threadIdx.x;
+  if (e >= PN) return;
+  float* seg = sg.state + (long long)bh * sg.nseg * PN + e;
+  float S = seg[0];
+  for (int s = 1; s < sg.nseg; ++s) {
+    const float local = seg[(long long)s * PN];
+    seg[(long long)s * PN] = S;
+    S = fmaf(sg.decay[(long long)bh * sg.nseg + s], S, local);
+  }
+  state[((long long)seq_slot[b] * heads + h) * PN + e] = S;
+}
+
 
 // Gated delta rule: S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q, with q and k made unit
 // vectors (x / sqrt(sum x^2 + unit_eps)), q times q_scale, beta = sigmoid(raw), g = exp(-exp(A_log) softplus(raw + bias)).
@@ -624,26 +677,57 @@ extern "C" int lq_causal_conv(const float* x, int ldx, const float* w, const flo
     default: LAUNCH(64, 16); break;          \
   }
 
+// Whether a launch over `batch` sequences, the longest bringing `max_rows` rows, runs in segments, and then the
+// float32 scratch it needs: one decision for the query and the launch.
+static long long ssd_segment_floats(int batch, int heads, int P, int N, int max_rows) {
+  ScanLaunch cfg;
+  if (max_rows < SEG_MIN_ROWS || !scan_launch(N, P, cfg)) return 0;
+  if ((long long)batch * heads * lq_ceil_div(P, cfg.cols) >= 4ll * lq_compute_units()) return 0;  // the chip is full as it is
+  return (long long)batch * heads * SEG_COUNT * ((long long)P * N + 1);
+}
+
+extern "C" long long lq_ssd_scan_workspace(int batch, int heads, int P, int N, int max_rows) {
+  if (batch <= 0 || heads <= 0 || P <= 0 || N <= 0) return 0;
+  return ssd_segment_floats(batch, heads, P, N, max_rows);
+}
+
 // x [rows, heads * P], B and C [rows, groups * N], dt [rows, heads] (before its softplus), state
-// [slots, heads, P, N], y [rows, heads * P]; rows lie sequence by sequence (cu_rows).
+// [slots, heads, P, N], y [rows, heads * P]; rows lie sequence by sequence (cu_rows).  `max_rows`: the most rows a
+// sequence brings (0: unknown); `scratch`: lq_ssd_scan_workspace(...) floats, or null (then no segments).
 extern "C" int lq_ssd_scan(const float* x, int ldx, const float* Bm, int ldb, const float* Cm, int ldc, const float* dt,
                            int lddt, const float* dt_bias, const float* a_log, const float* d_skip, float* state, float* y,
                            int ldy, int heads, int P, int N, int groups, const int* seq_slot, const int* cu_rows, int batch,
-                           hipStream_t stream) {
+                           int max_rows, float* scratch, long long scratch_floats, hipStream_t stream) {
   LQ_REQUIRE(heads > 0 && P > 0 && N > 0 && groups > 0 && heads % groups == 0 && batch > 0, "ssd_scan: bad sizes");
   LQ_REQUIRE(ldx >= heads * P && ldy >= heads * P && ldb >= groups * N && ldc >= groups * N && lddt >= heads,
              "ssd_scan: a row stride is smaller than its row");
   LQ_REQUIRE(x && Bm && Cm && dt && dt_bias && a_log && d_skip && state && y && seq_slot && cu_rows, "ssd_scan: null pointer");
   ScanLaunch cfg;
   LQ_REQUIRE(scan_launch(N, P, cfg), "ssd_scan: state size %d is too large", N);
-  dim3 grid((unsigned)(batch * heads), lq_ceil_div(P, cfg.cols));
+  const long long need = scratch != nullptr ? ssd_segment_floats(batch, heads, P, N, max_rows) : 0;
+  LQ_REQUIRE(need <= scratch_floats, "ssd_scan: %lld floats of scratch for a launch in segments, %lld given", need, scratch_floats);
+  SegArgs sg = {1, 1, nullptr, nullptr};
+  if (need > 0) {
+    sg.nseg = SEG_COUNT;
+    sg.state = scratch;
+    sg.decay = scratch + (long long)batch * heads * SEG_COUNT * P * N;
+  }
   ScanShape sh = {heads, groups, P, N, seq_slot, cu_rows};
 #define LQ_SSD(LN, SL)                                                                                              \
   ssd_scan_kernel<LN, SL><<<grid, cfg.threads, cfg.lds, stream>>>(x, ldx, Bm, ldb, Cm, ldc, dt, lddt, dt_bias, a_log, \
-                                                                  d_skip, state, y, ldy, sh)
+                                                                  d_skip, state, y, ldy, sh, sg)
+  dim3 grid((unsigned)(batch * heads), lq_ceil_div(P, cfg.cols), sg.nseg);
   LQ_SCAN_LANES(LQ_SSD)
-#undef LQ_SSD
   LQ_CHECK_LAUNCH("ssd_scan");
+  if (sg.nseg > 1) {
+    ssd_chain_kernel<<<dim3((unsigned)(batch * heads), lq_ceil_div(P * N, 256)), 256, 0, stream>>>(state, heads, P * N, sg,
+                                                                                               seq_slot, cu_rows);
+    LQ_CHECK_LAUNCH("ssd_scan(chain)");
+    sg.pass = 2;
+    LQ_SCAN_LANES(LQ_SSD)
+    LQ_CHECK_LAUNCH("ssd_scan(second pass)");
+  }
+#undef LQ_SSD
   return 0;
 }
 

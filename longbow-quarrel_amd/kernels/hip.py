@@ -799,13 +799,21 @@ class HipKernels:
                                             _ptr(seq_slot), _ptr(seq_start), _ptr(cu_rows), c_int(batch),
                                             c_int(self._ACTIVATIONS[activation]), self.stream))
 
+    @query
+    def ssd_scan_workspace(self, batch: int, heads: int, head_dim: int, n_state: int, max_rows: int) -> int:
+        """Float32 entries of scratch with which `ssd_scan` runs this launch in segments (0: it does not)."""
+        self.lib.lq_ssd_scan_workspace.restype = c_longlong
+        return int(self.lib.lq_ssd_scan_workspace(c_int(batch), c_int(heads), c_int(head_dim), c_int(n_state),
+                                                  c_int(max_rows)))
+
     def ssd_scan(self, x: torch.Tensor, b_in: torch.Tensor, c_in: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor,
                  a_log: torch.Tensor, d_skip: torch.Tensor, state: torch.Tensor, y: torch.Tensor, heads: int,
                  head_dim: int, n_state: int, groups: int, seq_slot: torch.Tensor, cu_rows: torch.Tensor,
-                 batch: int) -> None:
+                 batch: int, max_rows: int = 0, workspace: Optional[torch.Tensor] = None) -> None:
         """The Mamba-2 recurrence along every sequence of the step, token by token: with dt = softplus(dt + dt_bias),
         S <- exp(-exp(a_log) dt) S + dt B x^T and y = S^T C + d_skip x per head; state [slots, heads, head_dim,
-        n_state] is read and left at the step's end.  All float32."""
+        n_state] is read and left at the step's end.  All float32.  `max_rows` (the most rows a sequence brings)
+        and `workspace` (`ssd_scan_workspace(...)` floats) let a launch of few long sequences run in segments."""
         rows = x.shape[0]
         for t, what, cols in ((x, "x", heads * head_dim), (b_in, "B", groups * n_state), (c_in, "C", groups * n_state),
                               (dt, "dt", heads), (y, "y", heads * head_dim)):
@@ -819,12 +827,15 @@ class HipKernels:
             raise KernelLibraryError("ssd_scan: state must be dense [slots, heads, head_dim, n_state]")
         self._i32(seq_slot, "seq_slot", batch)
         self._i32(cu_rows, "cu_rows", batch + 1)
+        if workspace is not None:
+            self._f32(workspace, "ssd_scan: workspace", workspace.numel())
         ld = self._rows2d
         self._check(self.lib.lq_ssd_scan(_ptr(x), c_int(ld(x, "x")), _ptr(b_in), c_int(ld(b_in, "B")), _ptr(c_in),
                                          c_int(ld(c_in, "C")), _ptr(dt), c_int(ld(dt, "dt")), _ptr(dt_bias), _ptr(a_log),
                                          _ptr(d_skip), _ptr(state), _ptr(y), c_int(ld(y, "y")), c_int(heads),
                                          c_int(head_dim), c_int(n_state), c_int(groups), _ptr(seq_slot), _ptr(cu_rows),
-                                         c_int(batch), self.stream))
+                                         c_int(batch), c_int(max_rows if workspace is not None else 0), _ptr(workspace),
+                                         c_longlong(0 if workspace is None else workspace.numel()), self.stream))
 
     def delta_scan(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, beta: torch.Tensor, a: torch.Tensor,
                    dt_bias: torch.Tensor, a_log: torch.Tensor, state: torch.Tensor, out: torch.Tensor, heads: int,

@@ -107,9 +107,13 @@ class Mamba2(_Recurrent):
                        ctx.row_pos, ctx.row_seq, ctx.seq_slot, ctx.seq_start, ctx.seq_len, ctx.cu_rows, ctx.batch,
                        activation="silu")
         y = ctx.ws.alloc((rows, self.inner), torch.float32)
+        # a few long prompts: the kernel may cut them into segments that run side by side, given scratch
+        ask = getattr(kn, "ssd_scan_workspace", None)
+        need = ask(ctx.batch, self.heads, self.head_dim, self.state, ctx.max_new) if ask is not None else 0
+        more = dict(max_rows=ctx.max_new, workspace=ctx.ws.alloc((need,), torch.float32)) if need else {}
         kn.ssd_scan(xbc[:, : self.inner], xbc[:, self.inner : self.inner + gn], xbc[:, self.inner + gn :], dt,
                     self.dt_bias, self.a_log, self.d, state, y, self.heads, self.head_dim, self.state, self.groups,
-                    ctx.seq_slot, ctx.cu_rows, ctx.batch)
+                    ctx.seq_slot, ctx.cu_rows, ctx.batch, **more)
         normed = ctx.ws.alloc((rows, self.inner), ctx.dtype)
         kn.gated_rmsnorm(y, z, self.norm_w, self.eps, self.inner // self.norm_groups, normed, gate_first=True)
         if out is None:

@@ -175,6 +175,38 @@ def test_state_space_scan_in_portions(kn, sizes):
     assert torch.equal(y2[10:], torch.cat(got))
 
 
+def test_state_space_scan_of_a_long_prompt_in_segments(kn):
+    """A long sequence beside a short one: the long one is cut into segments that run side by side (given scratch);
+    results and the state left behind equal the plain recurrence, and the same launch without scratch."""
+    H, P, N, G = 3, 32, 48, 1
+    T, T2 = 1100, 37
+    x, B, C, dt = rnd(T, H, P, seed=1), rnd(T, G, N, seed=2, std=0.5), rnd(T, G, N, seed=3, std=0.5), rnd(T, H, seed=4)
+    dt_bias, a_log, d_skip = rnd(H, seed=5), rnd(H, seed=6, std=0.7) - 1.0, rnd(H, seed=7)
+    want = pv.ssd_scan(x.double(), B.double(), C.double(), pv.softplus(dt.double() + dt_bias.double()),
+                       a_log.double(), d_skip.double()).reshape(T, H * P)
+    cat = lambda t: dev(torch.cat([t[:T2], t]).reshape(T + T2, -1))
+    need = kn.ssd_scan_workspace(2, H, P, N, T)
+    assert need > 0 and kn.ssd_scan_workspace(2, H, P, N, 511) == 0
+    outs, states = [], []
+    for scratch in (torch.zeros(need, device=DEV), None):
+        state = torch.zeros((3, H, P, N), device=DEV)
+        y = torch.zeros((T + T2, H * P), device=DEV)
+        kn.ssd_scan(cat(x), cat(B), cat(C), cat(dt), dev(dt_bias), dev(a_log), dev(d_skip), state, y, H, P, N, G,
+                    i32([2, 0]), i32([0, T2, T + T2]), 2, max_rows=T, workspace=scratch)
+        assert vc.err(y[T2:], want) < 5e-6 and vc.err(y[:T2], want[:T2]) < 5e-6
+        outs.append(y)
+        states.append(state)
+    assert vc.err(states[0], states[1]) < 5e-6 and float(states[0][1].abs().max()) == 0.0
+    assert torch.equal(outs[0][:T2], outs[1][:T2])  # the short sequence runs whole either way
+    # ... and goes on from the state that the segments left
+    y = torch.zeros((1, H * P), device=DEV)
+    more = [rnd(1, H, P, seed=11), rnd(1, G, N, seed=12), rnd(1, G, N, seed=13), rnd(1, H, seed=14)]
+    for st in states:
+        kn.ssd_scan(*[dev(t.reshape(1, -1)) for t in more], dev(dt_bias), dev(a_log), dev(d_skip), st, y, H, P, N, G,
+                    i32([0]), i32([0, 1]), 1)
+    assert vc.err(states[0][0], states[1][0]) < 5e-6
+
+
 @pytest.mark.parametrize("sizes", [(4, 2, 16, 32), (2, 2, 48, 16), (2, 1, 24, 40), (3, 3, 128, 64), (1, 1, 272, 8), (3, 3, 12, 20),
                                    (1, 1, 520, 4)])
 def test_gated_delta_rule_scan_in_portions(kn, sizes):
@@ -296,6 +328,22 @@ def test_sizes_of_a_small_real_model(cases, dtype):
     t = vc.tokens(330, case.vocab, 6)
     for cuts in ([330], [290], [130, 70, 100]):
         assert vc.err(case.run_cut(t, cuts), case.want(t)) < tol(dtype), cuts
+    case.assert_idle()
+
+
+def test_a_prompt_long_enough_for_the_scan_in_segments_then_decoding(cases):
+    case = cases("a", "float32")
+    t = vc.tokens(700, case.vocab, 12)
+    assert vc.err(case.run_cut(t, [690]), case.want(t)) < TOL_F32
+    u = vc.tokens(40, case.vocab, 13)  # a long and a short request in one step
+    eng = case.eng
+    s1, s2 = eng.new_sequence(), eng.new_sequence()
+    out = eng.step([StepEntry(s1, u, range(40)), StepEntry(s2, t[:600], range(600))])
+    assert vc.err(out[:40], case.want(u)) < TOL_F32 and vc.err(out[40:], case.want(t)[:600]) < TOL_F32
+    out = eng.step([StepEntry(s2, t[600:], range(100))])
+    assert vc.err(out, case.want(t)[600:]) < TOL_F32
+    eng.release(s1)
+    eng.release(s2)
     case.assert_idle()
 
 
