@@ -15,8 +15,13 @@ from typing import Any, Dict, Optional, Tuple
 from .base import ConfigError, ModelConfig, coerce
 
 
-def _get(d: Dict[str, Any], key: str, where: str, kind=int, least=None):
+_REQUIRED = object()
+
+
+def _get(d: Dict[str, Any], key: str, where: str, kind=int, least=None, default=_REQUIRED):
     if not isinstance(d, dict) or key not in d or d[key] is None:
+        if default is not _REQUIRED and isinstance(d, dict):
+            return default  # what config.json does not mention, the model does not have
         raise ConfigError(f"config.json: required key '{where}.{key}' is missing")
     try:
         v = coerce(d[key], f"{where}.{key}", kind)
@@ -42,9 +47,11 @@ class AttentionSide:
         mask = d.get("mask") if isinstance(d, dict) else None
         if not isinstance(mask, dict):
             raise ConfigError(f"config.json: required key '{where}.mask' is missing")
-        c = cls(_get(d, "heads", where, least=1), _get(d, "kv_heads", where, least=1), _get(d, "dim", where, least=1),
-                _get(d, "vdim", where, least=1), _get(d, "scale", where, float), _get(mask, "size", where + ".mask", least=1),
-                _get(mask, "keep_first", where + ".mask", least=0))
+        heads = _get(d, "heads", where, least=1)
+        dim = _get(d, "dim", where, least=1)
+        c = cls(heads, _get(d, "kv_heads", where, least=1, default=heads), dim, _get(d, "vdim", where, least=1, default=dim),
+                _get(d, "scale", where, float), _get(mask, "size", where + ".mask", least=1),
+                _get(mask, "keep_first", where + ".mask", least=0, default=0))
         if c.heads % c.kv_heads:
             raise ConfigError(f"config.json: '{where}.heads' ({c.heads}) is no multiple of kv_heads ({c.kv_heads})")
         return c
@@ -66,7 +73,8 @@ class StateSpaceSide:
     @classmethod
     def from_dict(cls, d, where):
         c = cls(_get(d, "heads", where, least=1), _get(d, "vdim", where, least=1), _get(d, "state", where, least=1),
-                _get(d, "groups", where, least=1), _get(d, "conv", where, least=1), _get(d, "norm_groups", where, least=1))
+                _get(d, "groups", where, least=1, default=1), _get(d, "conv", where, least=1),
+                _get(d, "norm_groups", where, least=1, default=1))
         if c.heads % c.groups:
             raise ConfigError(f"config.json: '{where}.heads' ({c.heads}) is no multiple of groups ({c.groups})")
         if (c.heads * c.vdim) % c.norm_groups:
@@ -88,8 +96,10 @@ class DeltaMixer:
 
     @classmethod
     def from_dict(cls, d, where):
-        c = cls(_get(d, "heads", where, least=1), _get(d, "kv_heads", where, least=1), _get(d, "dim", where, least=1),
-                _get(d, "vdim", where, least=1), _get(d, "conv", where, least=1))
+        heads = _get(d, "heads", where, least=1)
+        dim = _get(d, "dim", where, least=1)
+        c = cls(heads, _get(d, "kv_heads", where, least=1, default=heads), dim, _get(d, "vdim", where, least=1, default=dim),
+                _get(d, "conv", where, least=1))
         if c.heads % c.kv_heads:
             raise ConfigError(f"config.json: '{where}.heads' ({c.heads}) is no multiple of kv_heads ({c.kv_heads})")
         return c

@@ -72,6 +72,24 @@ def test_configuration_errors_name_their_key(key, value, text):
     assert text in str(e.value)
 
 
+def test_keys_that_a_configuration_leaves_out_mean_that_the_model_has_no_such_thing():
+    cfg = copy.deepcopy(vc.CFG_A)
+    left, right = cfg["layers"][0]["mixer"]["left"], cfg["layers"][0]["mixer"]["right"]
+    del left["mask"]["keep_first"], left["kv_heads"], right["groups"], right["norm_groups"], cfg["layers"][1]["mlp"]
+    cfg["layers"][2] = copy.deepcopy(cfg["layers"][0])
+    cfg["layers"][2]["weights_of"] = 0
+    c = lq.VafodraConfig.from_dict(cfg)
+    assert c.layers[0].left.keep_first == 0 and c.layers[0].left.kv_heads == 4
+    assert c.layers[0].right.groups == 1 and c.layers[0].right.norm_groups == 1 and c.layers[1].ff is None
+
+
+def test_generation_with_delta_layers_alone(cases):
+    case = cases("f")
+    reqs, wants = vc.greedy(case, n_new=5, prompts=2)
+    res = lq.generate(case.eng, reqs, max_new_tokens=5, max_batch=2, stop_ids=[], use_graphs=False)
+    assert res.tokens == wants
+
+
 def test_weight_errors_list_missing_and_wrongly_shaped_tensors(tmp_path):
     w = vc.make_weights(vc.CFG_B, 1)
     del w["l1.mix.left.out"]
@@ -103,7 +121,7 @@ def test_a_window_that_keeps_first_tokens_gives_the_blocks_between_back():
     assert kept.blocks.taken_count == 0 and cm.free_blocks() == 6
 
 
-@pytest.mark.parametrize("name", ["a", "b", "c", "d"])
+@pytest.mark.parametrize("name", ["a", "b", "c", "d", "f"])
 def test_whole_prompts_and_token_by_token(cases, name):
     vc.whole_and_token_by_token(cases(name), TOL, lengths=(1, 2, 3, 70))
 

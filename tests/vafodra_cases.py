@@ -75,7 +75,12 @@ CFG_E = _config(1000, 512, 1.0, 1e-5, 0.5, [
     _parallel({"dim": 64, "vdim": 256, "heads": 2, "kv_heads": 2, "mask": {"size": 200, "keep_first": 0}, "scale": 0.125},
               {"conv": 4, "groups": 1, "heads": 16, "norm_groups": 1, "state": 64, "vdim": 32}, None),
 ])
-CONFIGS = {"a": CFG_A, "b": CFG_B, "c": CFG_C, "d": CFG_D, "e": CFG_E}
+# F: delta layers alone (no keys and values anywhere in the cache), the later layer lending its tensors to the earlier
+CFG_F = _config(50, 48, 1.2, 1e-5, 0.6, [
+    _delta({"conv": 3, "dim": 8, "heads": 6, "kv_heads": 2, "vdim": 8}, 24, weights_of=1),
+    _delta({"conv": 3, "dim": 8, "heads": 6, "kv_heads": 2, "vdim": 8}, 24),
+])
+CONFIGS = {"a": CFG_A, "b": CFG_B, "c": CFG_C, "d": CFG_D, "e": CFG_E, "f": CFG_F}
 
 
 def make_weights(cfg: dict, seed: int, sharp: float = 1.0) -> Dict[str, torch.Tensor]:
