@@ -31,7 +31,7 @@ __device__ inline f32x4 ld4(const bf16_t* p) {
 }
 
 struct SinkArgs {
-  int ldq, ldo, ldg, rows, rows_per_tile, nh, nkv, KD, VD;
+  int ldq, ldo, ldg, rows, rows_per_tile, heads_per_tile, nh, nkv, KD, VD;
   const int *row_pos, *row_seq, *seq_slot, *block_table;
   int bt_stride, BS;
   float scale;
@@ -65,11 +65,14 @@ __global__ __launch_bounds__(64 * SPLIT) void sink_tiles_kernel(const T* __restr
   constexpr int LDS_FLOATS = 64 * QROW > (SPLIT - 1) * PART ? 64 * QROW : (SPLIT - 1) * PART;
   __shared__ float smem[LDS_FLOATS];               // first the queries, at the end the partial results
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, c = lane & 15, g = lane >> 4;
-  const int h = blockIdx.y, kvh = h / (a.nh / a.nkv);
+  // The tile's 16 rows are rows_per_tile rows of the step times heads_per_tile query heads that share a kv head
+  // (tile row c: step row c / heads_per_tile, head c % heads_per_tile): their keys and values are read once.
+  const int GH = a.heads_per_tile;
+  const int hbase = blockIdx.y * GH, kvh = hbase / (a.nh / a.nkv);
   const int r0 = blockIdx.x * a.rows_per_tile;
   const int n_rows = min(a.rows_per_tile, a.rows - r0);
   const int HS = a.KD / 16, BS = a.BS;
-  const int my_row = r0 + min(c, n_rows - 1);
+  const int my_row = r0 + min(c / GH, n_rows - 1), h = hbase + c % GH;
   const int my_pos = a.row_pos[my_row], my_seq = a.row_seq[my_row];
   const int my_lo = (a.window > 0 && my_pos >= a.window) ? my_pos - a.window + 1 : 0;
   float* myq = smem + (g * 16 + c) * QROW;
@@ -92,7 +95,7 @@ __global__ __launch_bounds__(64 * SPLIT) void sink_tiles_kernel(const T* __restr
   const int seq_first = __builtin_amdgcn_readfirstlane(a.row_seq[r0]);
   const int seq_last = __builtin_amdgcn_readfirstlane(a.row_seq[r0 + n_rows - 1]);
   for (int seq = seq_first; seq <= seq_last; ++seq) {
-    const bool mine = my_seq == seq && c < n_rows;
+    const bool mine = my_seq == seq && c / GH < n_rows;
     int lo_min = mine ? my_lo : 0x7fffffff, pos_max = mine ? my_pos : -1;
 #pragma unroll
     for (int off = 1; off < 16; off <<= 1) {
@@ -220,11 +223,11 @@ __global__ __launch_bounds__(64 * SPLIT) void sink_tiles_kernel(const T* __restr
   for (int e = 0; e < 4; ++e) inv4[e] = __shfl(inv, 4 * g + e, 64);
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
-    const int row = 4 * g + e;
+    const int tr = 4 * g + e, row = tr / GH, hh = hbase + tr % GH;  // tile row -> step row and head
     if (row < n_rows) {
       float f = inv4[e];
-      if (gate != nullptr) f /= 1.f + expf(-to_f32(gate[(long long)(r0 + row) * a.ldg + h]));
-      T* orow = out + (long long)(r0 + row) * a.ldo + h * (HSV * 16) + c;
+      if (gate != nullptr) f /= 1.f + expf(-to_f32(gate[(long long)(r0 + row) * a.ldg + hh]));
+      T* orow = out + (long long)(r0 + row) * a.ldo + hh * (HSV * 16) + c;
 #pragma unroll
       for (int dt = 0; dt < HSV; ++dt) orow[dt * 16] = from_f32<T>(o[dt][e] * f);
     }
@@ -331,8 +334,11 @@ bool launch_tiles(const void* q, void* out, const void* gate, const void* kcache
       ((uintptr_t)q % (4 * el)) != 0 || ((uintptr_t)kcache % (4 * el)) != 0 || ((uintptr_t)vcache % (4 * el)) != 0)
     return false;
   SinkArgs b = a;
-  b.rows_per_tile = a.rows == batch ? 1 : 16;  // single tokens: a tile a row
-  dim3 grid(lq_ceil_div(a.rows, b.rows_per_tile), a.nh);
+  // the query heads of a kv head share a tile where their number is a power of two (or a multiple of 16)
+  const int group = a.nh / a.nkv;
+  b.heads_per_tile = group % 16 == 0 ? 16 : (group & (group - 1)) == 0 ? group : 1;
+  b.rows_per_tile = a.rows == batch ? 1 : 16 / b.heads_per_tile;  // single tokens: a tile a row of the step
+  dim3 grid(lq_ceil_div(a.rows, b.rows_per_tile), a.nh / b.heads_per_tile);
 #define LQ_SINK(HSV)                                                                                                  \
   case HSV:                                                                                                           \
     sink_tiles_kernel<T, HSV><<<grid, 64 * SPLIT, 0, stream>>>((const T*)q, (T*)out, (const T*)gate, (const T*)kcache,        \
@@ -381,7 +387,7 @@ extern "C" int lq_sink_attention(const void* q, int ldq, void* out, int ldo, con
   LQ_REQUIRE(q && out && row_pos && row_seq && seq_slot && block_table && kcache && vcache, "sink_attention: null pointer");
   LQ_REQUIRE(dtype == LQ_F32 || dtype == LQ_BF16, "sink_attention: unknown dtype %d", dtype);
   SinkArgs a;
-  a.ldq = ldq, a.ldo = ldo, a.ldg = ldg, a.rows = rows, a.rows_per_tile = 1, a.nh = nh, a.nkv = nkv, a.KD = KD, a.VD = VD;
+  a.ldq = ldq, a.ldo = ldo, a.ldg = ldg, a.rows = rows, a.rows_per_tile = 1, a.heads_per_tile = 1, a.nh = nh, a.nkv = nkv, a.KD = KD, a.VD = VD;
   a.row_pos = row_pos, a.row_seq = row_seq, a.seq_slot = seq_slot, a.block_table = block_table;
   a.bt_stride = bt_stride, a.BS = block_size, a.scale = scale, a.window = window, a.keep_first = keep_first, a.sink = sink;
   if (!force_rows) {
