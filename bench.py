@@ -155,7 +155,8 @@ def design_run(args) -> int:
             slots[0] = engine.new_sequence()
             timed.reset()
             engine.step([StepEntry(slots[0], prompt(n_prefill), [n_prefill - 1])])
-            by_op["prefill"] = {op: round(ms / layers * 1e3, 1) for op, (calls, ms) in timed.report().items()}
+            # (microseconds a call, calls a step)
+            by_op["prefill"] = {op: [round(ms / calls * 1e3, 1), calls] for op, (calls, ms) in timed.report().items()}
             engine.release(slots[0])
             slots[0] = engine.new_sequence()
             engine.step([StepEntry(s, prompt(prompt_len), [prompt_len - 1]) for s in slots])
@@ -163,11 +164,11 @@ def design_run(args) -> int:
             timed.reset()
             for _ in range(8):
                 engine.step([StepEntry(s, [1], [0]) for s in slots])
-            by_op["decode"] = {op: round(ms / 8 / layers * 1e3, 1) for op, (calls, ms) in timed.report().items()}
+            by_op["decode"] = {op: [round(ms / calls * 1e3, 1), calls // 8] for op, (calls, ms) in timed.report().items()}
             line = {"design": name, "width": width, "layers": layers, "prefill_tokens": n_prefill,
                     "prefill_ms": round(prefill_ms, 3), "prefill_tok_s": round(n_prefill / prefill_ms * 1e3, 1),
                     "decode_batch": batch, "decode_ms_per_step": round(step_ms, 4),
-                    "decode_tok_s": round(batch / step_ms * 1e3, 1), "us_per_layer_by_operation": by_op}
+                    "decode_tok_s": round(batch / step_ms * 1e3, 1), "us_per_call_and_calls_per_step": by_op}
             print(f"[bench] {json.dumps(line)}", file=sys.stderr, flush=True)
             results.append(line)
             del engine, backend, timed

@@ -168,19 +168,19 @@ struct ScanShape {
 
 // The chunk-wise staging that both scans share.  `a`, `b`: the two shared rows of a token ([rows, groups * N] each),
 // `x`: the per-column input ([rows, heads * P]).  LDS of one buffer: [TT][2 N] then [TT][cols] then [TT][2].
-template <int LN, int SLAB>
+template <int LN, int SLAB, int TH>  // TH: threads a workgroup
 struct Stage {
-  // entries of a token's two shared rows a thread of 256 (2 N <= 2 SLAB LN)
-  static constexpr int PER = 2 * SLAB * LN > 256 ? 2 * SLAB * LN / 256 : 1;
-  static constexpr int TT = PRE / PER;  // tokens a chunk
+  // entries of a token's two shared rows a thread (2 N <= 2 SLAB LN)
+  static constexpr int PER = 2 * SLAB * LN > TH ? 2 * SLAB * LN / TH : 1;
+  static constexpr int TT = PRE / PER;                    // tokens a chunk
   static constexpr int XPRE = TT / LN > 0 ? TT / LN : 1;  // chunk * cols / threads at most
   float ab[PRE];
   float xs[XPRE];
   float s0, s1;
 };
 
-template <int LN, int SLAB>
-__global__ __launch_bounds__(256, 2) void ssd_scan_kernel(const float* __restrict__ x, int ldx,
+template <int LN, int SLAB, int TH>
+__global__ __launch_bounds__(TH) void ssd_scan_kernel(const float* __restrict__ x, int ldx,
                                                        const float* __restrict__ Bm, int ldb,
                                                        const float* __restrict__ Cm, int ldc,
                                                        const float* __restrict__ dt, int lddt,
@@ -190,7 +190,7 @@ __global__ __launch_bounds__(256, 2) void ssd_scan_kernel(const float* __restric
                                                        float* __restrict__ y, int ldy, ScanShape sh, SegArgs sg) {
   extern __shared__ float lds[];
   const int heads = sh.heads, P = sh.P, N = sh.N;
-  constexpr int TT = Stage<LN, SLAB>::TT, PER = Stage<LN, SLAB>::PER;
+  constexpr int TT = Stage<LN, SLAB, TH>::TT, PER = Stage<LN, SLAB, TH>::PER;
   const int b = blockIdx.x / heads, h = blockIdx.x % heads, g = h / (heads / sh.groups);
   const int threads = blockDim.x, cols = threads / LN, tid = threadIdx.x;
   const int l = tid % LN, col = tid / LN, p0 = blockIdx.y * cols, p = p0 + col;
@@ -223,7 +223,7 @@ __global__ __launch_bounds__(256, 2) void ssd_scan_kernel(const float* __restric
     S[i] = (live && !from_zero && i < slab && n < N) ? from[n] : 0.f;
   }
   const float A = -expf(a_log[h]), bias = dt_bias[h], D = d_skip[h];
-  Stage<LN, SLAB> st;
+  Stage<LN, SLAB, TH> st;
 
   auto fetch = [&](long long c0, int nt) {  // the chunk's loads, into registers
 #pragma unroll
@@ -235,7 +235,7 @@ __global__ __launch_bounds__(256, 2) void ssd_scan_kernel(const float* __restric
           st.ab[t * PER + jj] = j < N ? Bm[(c0 + t) * ldb + g * N + j] : Cm[(c0 + t) * ldc + g * N + j - N];
       }
 #pragma unroll
-    for (int i = 0; i < Stage<LN, SLAB>::XPRE; ++i) {
+    for (int i = 0; i < Stage<LN, SLAB, TH>::XPRE; ++i) {
       const int e = tid + i * threads;
       if (e < nt * cols) {
         const int t = e / cols, c = e - t * cols;
@@ -253,7 +253,7 @@ __global__ __launch_bounds__(256, 2) void ssd_scan_kernel(const float* __restric
         if (t < nt && c < 2 * N) buf[t * 2 * NP + (c < N ? c : NP + c - N)] = st.ab[t * PER + jj];
       }
 #pragma unroll
-    for (int i = 0; i < Stage<LN, SLAB>::XPRE; ++i) {
+    for (int i = 0; i < Stage<LN, SLAB, TH>::XPRE; ++i) {
       const int e = tid + i * threads;
       if (e < nt * cols) buf[TT * 2 * NP + e] = st.xs[i];
     }
@@ -301,18 +301,22 @@ __global__ __launch_bounds__(256, 2) void ssd_scan_kernel(const float* __restric
     auto compute = [&](const Tok& k, int t) {
       const float dx = k.step * k.x;
       dprod *= k.decay;
-      float acc = 0.f;
+      float acc = 0.f, acc1 = 0.f;  // (two chains of multiply-adds, even and odd entries, added at the end)
 #pragma unroll
-      for (int i = 0; i < SLAB; ++i) {
+      for (int i = 0; i < SLAB; i += 2) {
         S[i] = fmaf(k.b[i], dx, k.decay * S[i]);
+        S[i + 1] = fmaf(k.b[i + 1], dx, k.decay * S[i + 1]);
         acc = fmaf(S[i], k.c[i], acc);
+        acc1 = fmaf(S[i + 1], k.c[i + 1], acc1);
       }
-      acc = group_sum<LN>(acc);
+      acc = group_sum<LN>(acc + acc1);
       if (l == 0) outs[t * cols + col] = fmaf(D, k.x, acc);
     };
     Tok ka, kb;
     load(ka, 0);
-    for (int t = 0; t < nt; t += 2) {
+#pragma unroll
+    for (int t = 0; t < TT; t += 2) {  // (unrolled: a token's places in LDS are constants)
+      if (t >= nt) break;
       if (t + 1 < nt) load(kb, t + 1);
       compute(ka, t);
       if (t + 1 < nt) {
@@ -358,22 +362,33 @@ __global__ __launch_bounds__(256) void ssd_chain_kernel(float* __restrict__ stat
 }
 
 
-// Gated delta rule: S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q, with q and k made unit
-// vectors (x / sqrt(sum x^2 + unit_eps)), q times q_scale, beta = sigmoid(raw), g = exp(-exp(A_log) softplus(raw + bias)).
+// q and k of every (row, q/k head) made unit vectors in place, x / sqrt(sum x^2 + eps), q also times q_scale: one
+// wavefront a (row, head), ahead of the scan (nothing of it depends on the state).
+__global__ __launch_bounds__(64) void unit_heads_kernel(float* __restrict__ q, int ldq, float* __restrict__ k, int ldk,
+                                                        int D, float q_scale, float eps) {
+  float* qr = q + (long long)blockIdx.x * ldq + blockIdx.y * D;
+  float* kr = k + (long long)blockIdx.x * ldk + blockIdx.y * D;
+  float sq = 0.f, sk = 0.f;
+  for (int d = threadIdx.x; d < D; d += 64) sq = fmaf(qr[d], qr[d], sq), sk = fmaf(kr[d], kr[d], sk);
+  const float qinv = q_scale / sqrtf(wave_sum(sq) + eps), kinv = 1.f / sqrtf(wave_sum(sk) + eps);
+  for (int d = threadIdx.x; d < D; d += 64) qr[d] *= qinv, kr[d] *= kinv;
+}
+
+// Gated delta rule: S <- g S;  u = beta (v - S^T k);  S <- S + k u^T;  o = S^T q, with q and k unit vectors (made so
+// by the kernel above), beta = sigmoid(raw), g = exp(-exp(A_log) softplus(raw + bias)).
 // (ScanShape: groups = q/k heads, N = key size.)
-template <int LN, int SLAB>
-__global__ __launch_bounds__(256, 2) void delta_scan_kernel(const float* __restrict__ q, int ldq,
+template <int LN, int SLAB, int TH>
+__global__ __launch_bounds__(TH) void delta_scan_kernel(const float* __restrict__ q, int ldq,
                                                          const float* __restrict__ k, int ldk,
                                                          const float* __restrict__ v, int ldv,
                                                          const float* __restrict__ beta, int ldbeta,
                                                          const float* __restrict__ a, int lda,
                                                          const float* __restrict__ dt_bias,
                                                          const float* __restrict__ a_log, float* __restrict__ state,
-                                                         float* __restrict__ out, int ldo, float q_scale,
-                                                         float unit_eps, ScanShape sh) {
+                                                         float* __restrict__ out, int ldo, ScanShape sh) {
   extern __shared__ float lds[];
   const int heads = sh.heads, P = sh.P, N = sh.N;
-  constexpr int TT = Stage<LN, SLAB>::TT, PER = Stage<LN, SLAB>::PER;
+  constexpr int TT = Stage<LN, SLAB, TH>::TT, PER = Stage<LN, SLAB, TH>::PER;
   const int b = blockIdx.x / heads, h = blockIdx.x % heads, j = h / (heads / sh.groups);
   const int threads = blockDim.x, cols = threads / LN, tid = threadIdx.x;
   const int l = tid % LN, col = tid / LN, p0 = blockIdx.y * cols, p = p0 + col;
@@ -390,7 +405,7 @@ __global__ __launch_bounds__(256, 2) void delta_scan_kernel(const float* __restr
     S[i] = (live && i < slab && n < N) ? sp[n] : 0.f;
   }
   const float A = -expf(a_log[h]), bias = dt_bias[h];
-  Stage<LN, SLAB> st;
+  Stage<LN, SLAB, TH> st;
 
   auto fetch = [&](long long c0, int nt) {
 #pragma unroll
@@ -402,7 +417,7 @@ __global__ __launch_bounds__(256, 2) void delta_scan_kernel(const float* __restr
           st.ab[t * PER + jj] = c < N ? q[(c0 + t) * ldq + j * N + c] : k[(c0 + t) * ldk + j * N + c - N];
       }
 #pragma unroll
-    for (int i = 0; i < Stage<LN, SLAB>::XPRE; ++i) {
+    for (int i = 0; i < Stage<LN, SLAB, TH>::XPRE; ++i) {
       const int e = tid + i * threads;
       if (e < nt * cols) {
         const int t = e / cols, c = e - t * cols;
@@ -423,7 +438,7 @@ __global__ __launch_bounds__(256, 2) void delta_scan_kernel(const float* __restr
         if (t < nt && c < 2 * N) buf[t * 2 * NP + (c < N ? c : NP + c - N)] = st.ab[t * PER + jj];
       }
 #pragma unroll
-    for (int i = 0; i < Stage<LN, SLAB>::XPRE; ++i) {
+    for (int i = 0; i < Stage<LN, SLAB, TH>::XPRE; ++i) {
       const int e = tid + i * threads;
       if (e < nt * cols) buf[TT * 2 * NP + e] = st.xs[i];
     }
@@ -465,29 +480,31 @@ __global__ __launch_bounds__(256, 2) void delta_scan_kernel(const float* __restr
       for (int i = 0; i < SLAB; ++i) k.q[i] = buf[t * 2 * NP + i * LN + l], k.k[i] = buf[t * 2 * NP + NP + i * LN + l];
     };
     auto compute = [&](const Tok& k, int t) {
-      float ssq = 0.f, ssk = 0.f, sk = 0.f;
+      float sk = 0.f, sk1 = 0.f;  // (two chains, even and odd entries)
 #pragma unroll
-      for (int i = 0; i < SLAB; ++i) {
-        ssk = fmaf(k.k[i], k.k[i], ssk);
-        ssq = fmaf(k.q[i], k.q[i], ssq);
+      for (int i = 0; i < SLAB; i += 2) {
         S[i] *= k.decay;
-        sk = fmaf(S[i], k.k[i], sk);  // with k as it came: the unit norm is one factor of the sum
+        S[i + 1] *= k.decay;
+        sk = fmaf(S[i], k.k[i], sk);
+        sk1 = fmaf(S[i + 1], k.k[i + 1], sk1);
       }
-      const float kinv = 1.f / sqrtf(group_sum<LN>(ssk) + unit_eps);
-      const float qinv = q_scale / sqrtf(group_sum<LN>(ssq) + unit_eps);
-      const float uk = k.beta * (k.v - group_sum<LN>(sk) * kinv) * kinv;
-      float o = 0.f;
+      const float u = k.beta * (k.v - group_sum<LN>(sk + sk1));
+      float o = 0.f, o1 = 0.f;
 #pragma unroll
-      for (int i = 0; i < SLAB; ++i) {
-        S[i] = fmaf(k.k[i], uk, S[i]);
+      for (int i = 0; i < SLAB; i += 2) {
+        S[i] = fmaf(k.k[i], u, S[i]);
+        S[i + 1] = fmaf(k.k[i + 1], u, S[i + 1]);
         o = fmaf(S[i], k.q[i], o);
+        o1 = fmaf(S[i + 1], k.q[i + 1], o1);
       }
-      o = group_sum<LN>(o) * qinv;
+      o = group_sum<LN>(o + o1);
       if (l == 0) outs[t * cols + col] = o;
     };
     Tok ka, kb;
     load(ka, 0);
-    for (int t = 0; t < nt; t += 2) {
+#pragma unroll
+    for (int t = 0; t < TT; t += 2) {  // (unrolled: a token's places in LDS are constants)
+      if (t >= nt) break;
       if (t + 1 < nt) load(kb, t + 1);
       compute(ka, t);
       if (t + 1 < nt) {
@@ -573,15 +590,23 @@ struct ScanLaunch {
   size_t lds;
 };
 
-bool scan_launch(int N, int P, ScanLaunch& s) {
+bool scan_launch(int N, int P, long long work, ScanLaunch& s) {
+  // Workgroups of 256 threads, fewer where a head has fewer columns than they would hold.  (Smaller workgroups for
+  // launches that leave compute units idle were measured and are not taken: every workgroup stages the whole shared
+  // rows of its tokens, and a chunk of fewer tokens pays its barrier more often; `work`, the (sequence, head,
+  // segment) triples of the launch, is kept for that choice.)  Nothing of a token's arithmetic depends on the size.
+  (void)work;
   s.slab = N > 512 ? 16 : 8;
   s.ln = 1;
   while ((N + s.ln - 1) / s.ln > s.slab) s.ln <<= 1;
   if (s.ln > 64) return false;
-  const int per = 2 * s.slab * s.ln > 256 ? 2 * s.slab * s.ln / 256 : 1;  // as Stage<LN, SLAB> has them
+  s.threads = 256;
+  while (s.threads > 64 && s.threads / 2 >= s.ln && 2 * s.slab * s.ln <= PRE * (s.threads / 2) &&
+         s.threads / s.ln >= 2 * P)
+    s.threads >>= 1;
+  const int per = 2 * s.slab * s.ln > s.threads ? 2 * s.slab * s.ln / s.threads : 1;  // as Stage<LN, SLAB, TH> has them
   s.tt = PRE / per;
-  s.threads = (P * s.ln + 63) / 64 * 64;
-  if (s.threads > 256 || 2 * N > per * s.threads) s.threads = 256;  // (2 N <= 2 slab LN <= per * 256)
+  if (s.tt < 1) return false;
   s.cols = s.threads / s.ln;
   s.lds = 2 * (size_t)s.tt * (2 * s.ln * s.slab + 2 * s.cols + 2) * sizeof(float);  // (rows padded to LN * slab)
   return s.lds <= 64 * 1024;
@@ -665,23 +690,27 @@ extern "C" int lq_causal_conv(const float* x, int ldx, const float* w, const flo
   return 0;
 }
 
-#define LQ_SCAN_LANES(LAUNCH)                \
-  switch (cfg.slab == 16 ? 128 : cfg.ln) {   \
-    case 1: LAUNCH(1, 8); break;             \
-    case 2: LAUNCH(2, 8); break;             \
-    case 4: LAUNCH(4, 8); break;             \
-    case 8: LAUNCH(8, 8); break;             \
-    case 16: LAUNCH(16, 8); break;           \
-    case 32: LAUNCH(32, 8); break;           \
-    case 64: LAUNCH(64, 8); break;           \
-    default: LAUNCH(64, 16); break;          \
+#define LQ_SCAN_TH(LAUNCH, LN, SL)                                 \
+  if (cfg.threads == 256) LAUNCH(LN, SL, 256);                     \
+  else if (cfg.threads == 128) LAUNCH(LN, SL, 128);                \
+  else LAUNCH(LN, SL, 64)
+#define LQ_SCAN_LANES(LAUNCH)                                      \
+  switch (cfg.slab == 16 ? 128 : cfg.ln) {                         \
+    case 1: { LQ_SCAN_TH(LAUNCH, 1, 8); } break;                   \
+    case 2: { LQ_SCAN_TH(LAUNCH, 2, 8); } break;                   \
+    case 4: { LQ_SCAN_TH(LAUNCH, 4, 8); } break;                   \
+    case 8: { LQ_SCAN_TH(LAUNCH, 8, 8); } break;                   \
+    case 16: { LQ_SCAN_TH(LAUNCH, 16, 8); } break;                 \
+    case 32: { LQ_SCAN_TH(LAUNCH, 32, 8); } break;                 \
+    case 64: { LQ_SCAN_TH(LAUNCH, 64, 8); } break;                 \
+    default: { LQ_SCAN_TH(LAUNCH, 64, 16); } break;                \
   }
 
 // Whether a launch over `batch` sequences, the longest bringing `max_rows` rows, runs in segments, and then the
 // float32 scratch it needs: one decision for the query and the launch.
 static long long ssd_segment_floats(int batch, int heads, int P, int N, int max_rows) {
   ScanLaunch cfg;
-  if (max_rows < SEG_MIN_ROWS || !scan_launch(N, P, cfg)) return 0;
+  if (max_rows < SEG_MIN_ROWS || !scan_launch(N, P, 1ll << 40, cfg)) return 0;  // (as workgroups of 256 threads)
   if ((long long)batch * heads * lq_ceil_div(P, cfg.cols) >= 4ll * lq_compute_units()) return 0;  // the chip is full as it is
   return (long long)batch * heads * SEG_COUNT * ((long long)P * N + 1);
 }
@@ -702,9 +731,10 @@ extern "C" int lq_ssd_scan(const float* x, int ldx, const float* Bm, int ldb, co
   LQ_REQUIRE(ldx >= heads * P && ldy >= heads * P && ldb >= groups * N && ldc >= groups * N && lddt >= heads,
              "ssd_scan: a row stride is smaller than its row");
   LQ_REQUIRE(x && Bm && Cm && dt && dt_bias && a_log && d_skip && state && y && seq_slot && cu_rows, "ssd_scan: null pointer");
-  ScanLaunch cfg;
-  LQ_REQUIRE(scan_launch(N, P, cfg), "ssd_scan: state size %d is too large", N);
   const long long need = scratch != nullptr ? ssd_segment_floats(batch, heads, P, N, max_rows) : 0;
+  ScanLaunch cfg;
+  LQ_REQUIRE(scan_launch(N, P, (long long)batch * heads * (need > 0 ? SEG_COUNT : 1), cfg),
+             "ssd_scan: state size %d is too large", N);
   LQ_REQUIRE(need <= scratch_floats, "ssd_scan: %lld floats of scratch for a launch in segments, %lld given", need, scratch_floats);
   SegArgs sg = {1, 1, nullptr, nullptr};
   if (need > 0) {
@@ -713,8 +743,8 @@ extern "C" int lq_ssd_scan(const float* x, int ldx, const float* Bm, int ldb, co
     sg.decay = scratch + (long long)batch * heads * SEG_COUNT * P * N;
   }
   ScanShape sh = {heads, groups, P, N, seq_slot, cu_rows};
-#define LQ_SSD(LN, SL)                                                                                              \
-  ssd_scan_kernel<LN, SL><<<grid, cfg.threads, cfg.lds, stream>>>(x, ldx, Bm, ldb, Cm, ldc, dt, lddt, dt_bias, a_log, \
+#define LQ_SSD(LN, SL, TH)                                                                                              \
+  ssd_scan_kernel<LN, SL, TH><<<grid, cfg.threads, cfg.lds, stream>>>(x, ldx, Bm, ldb, Cm, ldc, dt, lddt, dt_bias, a_log, \
                                                                   d_skip, state, y, ldy, sh, sg)
   dim3 grid((unsigned)(batch * heads), lq_ceil_div(P, cfg.cols), sg.nseg);
   LQ_SCAN_LANES(LQ_SSD)
@@ -733,21 +763,25 @@ extern "C" int lq_ssd_scan(const float* x, int ldx, const float* Bm, int ldb, co
 
 // q and k [rows, kv_heads * Dk], v [rows, heads * P], beta and a [rows, heads] (raw), state [slots, heads, P, Dk],
 // out [rows, heads * P]
-extern "C" int lq_delta_scan(const float* q, int ldq, const float* k, int ldk, const float* v, int ldv, const float* beta,
+// (q and k are made unit vectors in place)
+extern "C" int lq_delta_scan(float* q, int ldq, float* k, int ldk, const float* v, int ldv, const float* beta,
                              int ldbeta, const float* a, int lda, const float* dt_bias, const float* a_log, float* state,
                              float* out, int ldo, int heads, int kv_heads, int Dk, int P, float q_scale, float unit_eps,
-                             const int* seq_slot, const int* cu_rows, int batch, hipStream_t stream) {
+                             const int* seq_slot, const int* cu_rows, int batch, int rows, hipStream_t stream) {
   LQ_REQUIRE(heads > 0 && kv_heads > 0 && heads % kv_heads == 0 && Dk > 0 && P > 0 && batch > 0, "delta_scan: bad sizes");
   LQ_REQUIRE(ldq >= kv_heads * Dk && ldk >= kv_heads * Dk && ldv >= heads * P && ldo >= heads * P && ldbeta >= heads &&
                  lda >= heads, "delta_scan: a row stride is smaller than its row");
   LQ_REQUIRE(q && k && v && beta && a && dt_bias && a_log && state && out && seq_slot && cu_rows, "delta_scan: null pointer");
   ScanLaunch cfg;
-  LQ_REQUIRE(scan_launch(Dk, P, cfg), "delta_scan: key size %d is too large", Dk);
+  LQ_REQUIRE(scan_launch(Dk, P, (long long)batch * heads, cfg), "delta_scan: key size %d is too large", Dk);
+  LQ_REQUIRE(rows > 0 && rows <= 0x7fffffff && kv_heads <= 65535, "delta_scan: %d rows, %d q/k heads", rows, kv_heads);
+  unit_heads_kernel<<<dim3((unsigned)rows, kv_heads), 64, 0, stream>>>(q, ldq, k, ldk, Dk, q_scale, unit_eps);
+  LQ_CHECK_LAUNCH("delta_scan(unit vectors)");
   dim3 grid((unsigned)(batch * heads), lq_ceil_div(P, cfg.cols));
   ScanShape sh = {heads, kv_heads, P, Dk, seq_slot, cu_rows};
-#define LQ_DELTA(LN, SL)                                                                                             \
-  delta_scan_kernel<LN, SL><<<grid, cfg.threads, cfg.lds, stream>>>(q, ldq, k, ldk, v, ldv, beta, ldbeta, a, lda,      \
-                                                                    dt_bias, a_log, state, out, ldo, q_scale, unit_eps, sh)
+#define LQ_DELTA(LN, SL, TH)                                                                                             \
+  delta_scan_kernel<LN, SL, TH><<<grid, cfg.threads, cfg.lds, stream>>>(q, ldq, k, ldk, v, ldv, beta, ldbeta, a, lda,      \
+                                                                    dt_bias, a_log, state, out, ldo, sh)
   LQ_SCAN_LANES(LQ_DELTA)
 #undef LQ_DELTA
   LQ_CHECK_LAUNCH("delta_scan");

@@ -844,7 +844,7 @@ class HipKernels:
         """The gated delta rule along every sequence of the step, token by token: q and k made unit vectors per
         head (x / sqrt(sum x^2 + unit_eps)), q times q_scale, beta = sigmoid(beta), g = exp(-exp(a_log)
         softplus(a + dt_bias)); S <- g S, u = beta (v - S^T k), S <- S + k u^T, out = S^T q.  state [slots, heads,
-        value_dim, key_dim].  All float32."""
+        value_dim, key_dim].  All float32.  q and k are overwritten with their unit vectors."""
         rows = q.shape[0]
         for t, what, cols in ((q, "q", kv_heads * key_dim), (k, "k", kv_heads * key_dim), (v, "v", heads * value_dim),
                               (beta, "beta", heads), (a, "a", heads), (out, "out", heads * value_dim)):
@@ -864,7 +864,7 @@ class HipKernels:
                                            c_int(ld(a, "a")), _ptr(dt_bias), _ptr(a_log), _ptr(state), _ptr(out),
                                            c_int(ld(out, "out")), c_int(heads), c_int(kv_heads), c_int(key_dim),
                                            c_int(value_dim), c_float(q_scale), c_float(unit_eps), _ptr(seq_slot),
-                                           _ptr(cu_rows), c_int(batch), self.stream))
+                                           _ptr(cu_rows), c_int(batch), c_int(rows), self.stream))
 
     def gated_rmsnorm(self, y: torch.Tensor, z: torch.Tensor, weight: torch.Tensor, eps: float, group: int,
                       out: torch.Tensor, gate_first: bool = True) -> None:
