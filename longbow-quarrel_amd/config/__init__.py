@@ -2,5 +2,6 @@
 from .base import ConfigError, ModelConfig, read_config_json
 from .llama import LlamaConfig, RopeScaling
 from .vafodra import VafodraConfig
+from .vupelorn import VupelornConfig
 
-__all__ = ["ConfigError", "ModelConfig", "read_config_json", "LlamaConfig", "RopeScaling", "VafodraConfig"]
+__all__ = ["ConfigError", "ModelConfig", "read_config_json", "LlamaConfig", "RopeScaling", "VafodraConfig", "VupelornConfig"]

@@ -28,6 +28,11 @@ class ModelConfig:
     def to_dict(self) -> Dict[str, Any]:
         raise NotImplementedError
 
+    def completed(self, shapes) -> "ModelConfig":
+        """The configuration with the sizes that no key of config.json gives, taken from the shapes of a model
+        file's tensors (`shapes`: name -> shape).  Most designs have none: the configuration itself."""
+        return self
+
 
 def read_config_json(folder: str) -> Dict[str, Any]:
     path = os.path.join(folder, "config.json")

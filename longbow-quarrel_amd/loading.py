@@ -11,7 +11,7 @@ from .engine.step import Engine
 from .model import DecoderModel
 from .parts.base import BuildEnv
 from .registry import config_from_dict, spec_from_config
-from .weights.loader import check_names_and_shapes, load_tensors
+from .weights.loader import check_names_and_shapes, load_tensors, tensor_shapes
 from .weights.random_init import random_tensors
 
 _DTYPES = {
@@ -44,7 +44,7 @@ def load_engine(folder: str, dtype: Union[str, torch.dtype] = "bfloat16", max_to
     """config.json chooses the model class; model.safetensors is bound by tensor name.
     `max_tokens` sizes the cache for all live sequences together; `max_sequence_tokens` bounds one
     sequence (default: what the configuration allows, `max_position_embeddings` for Llama)."""
-    config = config_from_dict(read_config_json(folder))
+    config = config_from_dict(read_config_json(folder)).completed(tensor_shapes(folder))
     model = DecoderModel(spec_from_config(config))
     env = _env(dtype, device, kernels)
     tensors = load_tensors(folder, model.tensor_specs(), env.dtype, env.device)

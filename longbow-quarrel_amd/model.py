@@ -24,6 +24,10 @@ from .parts.base import (BLOCKS, EMBEDDINGS, LOGIT_STEPS, MATRIX, NORMS, Block, 
                          project_normed)
 
 
+#: the key of the embedding's own per-sequence store among the cache needs and views (the runs count from 0)
+EMBEDDING_RUN = -1
+
+
 @dataclass(frozen=True)
 class Run:
     layer: int
@@ -123,8 +127,11 @@ class DecoderModel:
 
     # ---- what the cache has to hold -----------------------------------------------
     def cache_needs(self) -> Dict[int, object]:
-        """Run number -> KVNeed / StateNeed, for the runs of the schedule that own a cache."""
+        """Run number -> KVNeed / StateNeed, for the runs of the schedule that own a cache (and `EMBEDDING_RUN`
+        for an embedding that keeps something per sequence)."""
         needs = {}
+        if self.embedding.cache_need() is not None:
+            needs[EMBEDDING_RUN] = self.embedding.cache_need()
         for i, run in enumerate(self.spec.schedule):
             if run.cache_of is None:
                 need = self.blocks[run.layer].mixer.cache_need()
@@ -150,7 +157,8 @@ class DecoderModel:
         of the rows listed in want_rows (None when nothing is wanted)."""
         kn = ctx.kernels
         s = self.spec
-        x = self.embedding.forward(ctx)
+        x = self.embedding.forward(ctx, caches.get(EMBEDDING_RUN)) if EMBEDDING_RUN in caches \
+            else self.embedding.forward(ctx)
         pending: Optional[torch.Tensor] = None
         if ctx.observe is not None:
             ctx.observe("embed", x, None)

@@ -357,6 +357,11 @@ class Embedding(Part):
 
     table: Optional[torch.Tensor] = None
 
+    def cache_need(self):
+        """What the embedding keeps for every sequence between steps (a `CacheNeed`), or None.  An embedding with
+        a need is called as forward(ctx, cache)."""
+        return None
+
     def forward(self, ctx: StepContext) -> torch.Tensor:
         raise NotImplementedError
 

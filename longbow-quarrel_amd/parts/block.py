@@ -146,3 +146,90 @@ class ParallelBlock(Block):
                 kn.add(out, piece)
         else:
             kn.cast(got, out)
+
+
+class RoundedStream:
+    """What an `OutputNormBlock` leaves pending: the stream x is up to date, and `rounded` holds it in the run's
+    dtype, made by the kernel that added the last sublayer's result.  The next block of the same kind reads it
+    instead of rounding x again; anyone else has nothing to add (`settle`)."""
+
+    def __init__(self, rounded: torch.Tensor) -> None:
+        self.rounded = rounded
+
+    def settle(self, x: torch.Tensor, ctx: StepContext) -> None:
+        return None
+
+
+@BLOCKS.register("output_norm")
+class OutputNormBlock(Block):
+    """Norms on the sublayers' results, none on their inputs: x += norm1(mixer(x)); x += norm2(ffn(x)).  The
+    sublayers read the stream itself (rounded to the run's dtype where that is narrower).  The norms are RMS norms;
+    one kernel normalises a sublayer's result, adds it to the 32-bit stream and leaves the stream's rounding for the
+    next reader.  The feed-forward may be absent (`feed_forward=None`; then there is no second norm either)."""
+
+    def __init__(self, mixer: PartSpec, mixer_norm: PartSpec, feed_forward: Optional[PartSpec] = None,
+                 ffn_norm: Optional[PartSpec] = None) -> None:
+        self.mixer = build_part(MIXERS, mixer)
+        self.mixer_norm = build_part(NORMS, mixer_norm)
+        self.ffn = build_part(FEED_FORWARDS, feed_forward) if feed_forward is not None else None
+        self.ffn_norm = build_part(NORMS, ffn_norm) if feed_forward is not None else None
+        if feed_forward is not None and ffn_norm is None:
+            raise ValueError("a feed-forward needs the norm of its result")
+        for norm in (self.mixer_norm, self.ffn_norm):
+            if norm is not None and not getattr(norm, "deferrable", False):
+                raise ValueError("the norms on the sublayers' results must be RMS norms")
+
+    @property
+    def graph_safe(self) -> bool:
+        return all(p.graph_safe for p in self.parts())
+
+    def parts(self):
+        return tuple(p for p in (self.mixer, self.mixer_norm, self.ffn, self.ffn_norm) if p is not None)
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        return [s for p in self.parts() for s in p.tensor_specs()]
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], env: BuildEnv) -> None:
+        super().bind(tensors, env)
+        for p in self.parts():
+            p.bind(tensors, env)
+
+    @staticmethod
+    def _run(part, args, ctx: StepContext, width: int) -> torch.Tensor:
+        """A sublayer's result, whole [rows, width] in 32-bit."""
+        rows = args[0].shape[0]
+        if part.takes_out:
+            out = ctx.ws.alloc((rows, width), torch.float32)
+            part.forward(*args, out=out)
+            return out
+        got = part.forward(*args)
+        if got.dim() == 3 or got.dtype != torch.float32:
+            out = ctx.ws.alloc((rows, width), torch.float32)
+            ParallelBlock._copy_into(ctx.kernels, got, out)
+            return out
+        return got
+
+    def _add_normed(self, x, y, norm, ctx: StepContext):
+        """x += norm(y); -> x in the run's dtype."""
+        narrow = ctx.dtype != torch.float32
+        rounded = ctx.ws.alloc(x.shape, ctx.dtype) if narrow else None
+        ctx.kernels.rmsnorm_residual(x, y, norm.weight, norm.eps, rounded)
+        return rounded if narrow else x
+
+    def forward(self, x: torch.Tensor, pending, ctx: StepContext, cache: Optional[LayerCache]):
+        kn = ctx.kernels
+        if isinstance(pending, RoundedStream):
+            h = pending.rounded
+        else:
+            if hasattr(pending, "settle"):
+                pending = pending.settle(x, ctx)
+            if pending is not None and not isinstance(pending, RowStats):
+                kn.add(x, pending)
+            h = x
+            if ctx.dtype != torch.float32:
+                h = ctx.ws.alloc(x.shape, ctx.dtype)
+                kn.cast(x, h)
+        h = self._add_normed(x, self._run(self.mixer, (h, ctx, cache), ctx, x.shape[1]), self.mixer_norm, ctx)
+        if self.ffn is not None:
+            h = self._add_normed(x, self._run(self.ffn, (h, ctx), ctx, x.shape[1]), self.ffn_norm, ctx)
+        return RoundedStream(h) if h is not x else None

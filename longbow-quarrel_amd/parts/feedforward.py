@@ -116,3 +116,74 @@ class GatedLinearUnit(FeedForward):
             out = ctx.ws.alloc((rows, self.width), torch.float32)
         project(kn, ctx, act, self.w_down, out)
         return out
+
+
+@FEED_FORWARDS.register("moe")
+class MixtureOfExperts(FeedForward):
+    """`experts` small gated feed-forwards of which every token uses `top`, chosen by a router.
+
+    Router: z = Wr h in 32-bit, s = sigmoid(z); the `top` largest scores win (the lower index on a tie); an expert's
+    weight is its score as it is (`renormalize` divides the chosen scores by their sum).  With `weight_input` the
+    weight multiplies what the expert reads, out = sum_e expert_e(s_e h); otherwise its result.
+
+    Expert (`activation` "clamped_swish"): g = min(Wg h, limit), u = clamp(Wu h, -limit, limit),
+    y = g sigmoid(1.702 g) (u + 1), result Wd y; no biases.  Wg (s h) = s (Wg h), so the weight is applied to the
+    32-bit results of the gate and up products, ahead of the clamps.
+
+    How it runs.  The experts' gate and up matrices are one matrix [experts * 2 ff, width] and their down matrices
+    one [width, experts * ff]: with the activations of the experts that a token did not choose set to zero, the down
+    product adds the chosen experts' results by itself.  Every row runs through all experts' columns: a decoding
+    batch of more than a few tokens reads nearly all experts anyway; a prompt pays experts / top times the
+    arithmetic of a step whose rows are sorted by expert, which is not built."""
+
+    graph_safe = True
+    takes_out = True
+
+    def __init__(self, width: int, experts: int, top: int, inner: int, limit: float, prefix: str,
+                 weight_input: bool = True, renormalize: bool = False, names: Optional[Mapping[str, str]] = None) -> None:
+        self.width, self.experts, self.top, self.inner = int(width), int(experts), int(top), int(inner)
+        self.limit, self.weight_input, self.renormalize = float(limit), bool(weight_input), bool(renormalize)
+        if not 1 <= self.top <= self.experts:
+            raise ValueError(f"{top} of {experts} experts cannot be chosen")
+        n = {"router": "router", "expert": "e{}", "gate": "gate", "up": "up", "down": "down"}
+        n.update(names or {})
+        self.prefix, self.n = prefix, n
+
+    def _name(self, e: int, what: str) -> str:
+        return f"{self.prefix}.{self.n['expert'].format(e)}.{self.n[what]}"
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        specs = []
+        for e in range(self.experts):
+            specs += [TensorSpec(self._name(e, "gate"), (self.inner, self.width)),
+                      TensorSpec(self._name(e, "up"), (self.inner, self.width)),
+                      TensorSpec(self._name(e, "down"), (self.width, self.inner))]
+        return specs + [TensorSpec(f"{self.prefix}.{self.n['router']}", (self.experts, self.width))]
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], env: BuildEnv) -> None:
+        super().bind(tensors, env)
+        E = self.experts
+        gu = [tensors[self._name(e, w)] for e in range(E) for w in ("gate", "up")]
+        down = [tensors[self._name(e, "down")] for e in range(E)]
+        if len({m.dtype for m in gu + down}) != 1:
+            raise ValueError(f"{self._name(0, 'gate')}: the experts' matrices are stored in different dtypes")
+        # expert e's rows of the first matrix: [gate (ff) | up (ff)]; its columns of the second: e ff .. (e + 1) ff
+        self.w_gate_up = product_weight(env, torch.cat(gu, dim=0))  # [E * 2 ff, width]
+        self.w_down = product_weight(env, torch.cat(down, dim=1))   # [width, E * ff]
+        self.w_router = tensors[f"{self.prefix}.{self.n['router']}"].float().contiguous()  # the router is 32-bit
+
+    def forward(self, h, ctx: StepContext, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        kn = ctx.kernels
+        rows, E, ff = h.shape[0], self.experts, self.inner
+        z = ctx.ws.alloc((rows, (E + 3) // 4 * 4), torch.float32)[:, :E]
+        project(kn, ctx, h, self.w_router, z)
+        route = ctx.ws.alloc((rows, E), torch.float32)  # the weight of a chosen expert, -1 for the others
+        kn.moe_route(z, route, self.top, self.renormalize)
+        if out is None:
+            out = ctx.ws.alloc((rows, self.width), torch.float32)
+        gu = ctx.ws.alloc((rows, E * 2 * ff), torch.float32)
+        project(kn, ctx, h, self.w_gate_up, gu)
+        act = ctx.ws.alloc((rows, E * ff), ctx.dtype)
+        kn.moe_glu(gu, route, act, E, ff, self.limit, self.weight_input)
+        project(kn, ctx, act, self.w_down, out)
+        return out

@@ -268,3 +268,91 @@ class SideBySide(Mixer):
 
 def _need_or_nothing(need):
     return need if need is not None else MultiNeed(())
+
+
+@MIXERS.register("gated_linear_attention")
+class GatedLinearAttention(Mixer):
+    """Linear attention with a decay per key channel (Yang, Wang, Shen, Panda, Kim: "Gated Linear Attention
+    Transformers with Hardware-Efficient Training").  q and k are `heads` x `key_dim`, v is `heads` x `value_dim`;
+    q is scaled by key_dim^(-1/2).  The decay comes through a bottleneck of `decay_rank` columns:
+    a = sigmoid(W2 (W1 h) + b)^(1 / tau), one number for every key channel of every head.  Per head, with the state
+    S [key_dim, value_dim] starting at zero:
+
+        S <- diag(a) S + k v^T,      o = S^T q.
+
+    Each head's o is divided by its root mean square over value_dim and multiplied by a weight that the heads share,
+    then by silu of one more projection of the input; then the output projection.  The decay, its logarithm and the
+    state are 32-bit; one kernel walks prompts and single tokens alike, token by token."""
+
+    graph_safe = True
+    takes_out = True
+
+    def __init__(self, width: int, heads: int, key_dim: int, value_dim: int, decay_rank: int, tau: float, eps: float,
+                 prefix: str, names: Optional[Mapping[str, str]] = None) -> None:
+        self.width, self.heads, self.key_dim, self.value_dim = int(width), int(heads), int(key_dim), int(value_dim)
+        self.decay_rank, self.tau, self.eps = int(decay_rank), float(tau), float(eps)
+        if self.tau <= 0 or self.decay_rank < 1:
+            raise ValueError("the decay needs a positive tau and a rank of at least one")
+        self.qk_width, self.v_width = self.heads * self.key_dim, self.heads * self.value_dim
+        n = {"q": "q", "k": "k", "v": "v", "gate": "g", "a1": "a1", "a2": "a2", "a2_bias": "a2.b", "norm": "norm",
+             "o": "o"}
+        n.update(names or {})
+        self.names: Dict[str, str] = {key: f"{prefix}.{val}" for key, val in n.items()}
+
+    def tensor_specs(self) -> List[TensorSpec]:
+        nm = self.names
+        return [
+            TensorSpec(nm["q"], (self.qk_width, self.width)),
+            TensorSpec(nm["k"], (self.qk_width, self.width)),
+            TensorSpec(nm["v"], (self.v_width, self.width)),
+            TensorSpec(nm["gate"], (self.v_width, self.width)),
+            TensorSpec(nm["o"], (self.width, self.v_width)),
+            TensorSpec(nm["norm"], (self.value_dim,), kind=VECTOR32, init="around_one"),
+            TensorSpec(nm["a1"], (self.decay_rank, self.width)),
+            TensorSpec(nm["a2"], (self.qk_width, self.decay_rank)),
+            TensorSpec(nm["a2_bias"], (self.qk_width,), kind=VECTOR32),
+        ]
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], env: BuildEnv) -> None:
+        super().bind(tensors, env)
+        nm = self.names
+        mats = [tensors[nm[k]] for k in ("q", "k", "v", "gate")]
+        if len({m.dtype for m in mats}) != 1:
+            raise ValueError(f"{nm['q']}: the projections of one input are stored in different dtypes")
+        self.w_in = product_weight(env, torch.cat(mats, dim=0))  # [q | k | v | gate]: 32-bit results for the scan
+        # the bottleneck is a product of its own: its result feeds the next product in the run's dtype
+        self.w_a1 = product_weight(env, tensors[nm["a1"]])
+        self.w_a2 = product_weight(env, tensors[nm["a2"]])
+        self.w_o = product_weight(env, tensors[nm["o"]])
+        self.a2_bias, self.norm_w = tensors[nm["a2_bias"]].contiguous(), tensors[nm["norm"]].contiguous()
+
+    def cache_need(self) -> StateNeed:
+        # held [head, value_dim, key_dim]: a thread of the scan owns a run of one column's key channels
+        return StateNeed((self.heads, self.value_dim, self.key_dim), torch.float32)
+
+    def forward(self, h: torch.Tensor, ctx: StepContext, cache, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        kn = ctx.kernels
+        if cache is None or getattr(cache, "state", None) is None:
+            raise RuntimeError("gated linear attention needs its state")
+        if not cache.write:
+            raise RuntimeError("a recurrent state cannot be shared between runs of the schedule")
+        rows = h.shape[0]
+        qk, vw, rank = self.qk_width, self.v_width, self.decay_rank
+        total = 2 * qk + 2 * vw
+        u = ctx.ws.alloc((rows, _round4(total)), torch.float32)[:, :total]
+        project(kn, ctx, h, self.w_in, u)
+        low = ctx.ws.alloc((rows, (rank + 7) // 8 * 8), self.w_a2.dtype)[:, :rank]
+        project(kn, ctx, h, self.w_a1, low)
+        z = ctx.ws.alloc((rows, qk), torch.float32)
+        project(kn, ctx, low, self.w_a2, z)
+        o = ctx.ws.alloc((rows, vw), torch.float32)
+        kn.gla_scan(u[:, :qk], u[:, qk : 2 * qk], u[:, 2 * qk : 2 * qk + vw], z, self.a2_bias, cache.state, o,
+                    self.heads, self.key_dim, self.value_dim, self.key_dim ** -0.5, 1.0 / self.tau,
+                    ctx.seq_slot, ctx.cu_rows, ctx.batch)
+        normed = ctx.ws.alloc((rows, vw), ctx.dtype)
+        kn.gated_rmsnorm(o, u[:, 2 * qk + vw : 2 * qk + 2 * vw], self.norm_w, self.eps, self.value_dim, normed,
+                         gate_first=False)
+        if out is None:
+            out = ctx.ws.alloc((rows, self.width), torch.float32)
+        project(kn, ctx, normed, self.w_o, out)
+        return out

@@ -8,6 +8,12 @@ L_i = 2 pi / f_i, L_i < original / high_freq_factor keeps f_i,
 L_i > original / low_freq_factor gives f_i / factor, and between the two
 s = (original / L_i - low) / (high - low), f_i' = (1 - s) f_i / factor + s f_i.
 
+`yarn` (Peng, Quesnelle, Fan, Shippole: "YaRN: Efficient Context Window Extension of Large Language Models")
+blends per pair: with d(t) = dims ln(original / (2 pi t)) / (2 ln base) the pair index at which a wave turns t
+times within `original` positions, lo = max(floor(d(fast)), 0), hi = min(ceil(d(slow)), dims - 1) and
+r_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1): f_i' = r_i f_i / factor + (1 - r_i) f_i; cos and sin are
+also multiplied by 0.1 ln(factor) + 1 (`rotary_magnitude`).
+
 The table is computed once in float64 and handed to the kernel as a parameter,
 so the kernel knows nothing about scaling types.
 """
@@ -29,8 +35,18 @@ def rotary_frequencies(head_dim: int, base: float, scaling: Optional[Mapping] = 
     kind = scaling.get("rope_type", "llama3")
     if kind == "linear":  # positions divided by the factor
         return [f / factor for f in freqs]
+    if kind == "yarn":
+        original = float(scaling["original"])
+
+        def pair_of(turns: float) -> float:
+            return head_dim * math.log(original / (2.0 * math.pi * turns)) / (2.0 * math.log(base))
+
+        lo = max(math.floor(pair_of(float(scaling["fast"]))), 0)
+        hi = min(math.ceil(pair_of(float(scaling["slow"]))), head_dim - 1)
+        ramps = [min(1.0, max(0.0, (i - lo) / max(hi - lo, 0.001))) for i in range(head_dim // 2)]
+        return [f / factor * r + f * (1.0 - r) for f, r in zip(freqs, ramps)]
     if kind != "llama3":
-        raise ValueError(f"rope scaling type {kind!r} is not known (known: 'linear', 'llama3')")
+        raise ValueError(f"rope scaling type {kind!r} is not known (known: 'linear', 'llama3', 'yarn')")
     low = float(scaling["low_freq_factor"])
     high = float(scaling["high_freq_factor"])
     original = float(scaling["original_max_position_embeddings"])
@@ -45,6 +61,13 @@ def rotary_frequencies(head_dim: int, base: float, scaling: Optional[Mapping] = 
             s = (original / wavelen - low) / (high - low)
             out.append((1.0 - s) * f / factor + s * f)
     return out
+
+
+def rotary_magnitude(scaling: Optional[Mapping] = None) -> float:
+    """What cos and sin are multiplied by: 0.1 ln(factor) + 1 under `yarn` scaling, else 1."""
+    if scaling and scaling.get("rope_type", "llama3") == "yarn":
+        return 0.1 * math.log(float(scaling["factor"])) + 1.0
+    return 1.0
 
 
 @POSITION_ENCODINGS.register("rope")

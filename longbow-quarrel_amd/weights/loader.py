@@ -67,6 +67,17 @@ def check_names_and_shapes(specs: Sequence[TensorSpec], found: Mapping[str, tupl
         raise WeightError(where, sorted(missing), sorted(unexpected), sorted(wrong))
 
 
+def tensor_shapes(folder: str) -> Dict[str, tuple]:
+    """name -> shape of every tensor in the folder's files (headers only): for a configuration whose config.json
+    leaves a size to the tensors (`ModelConfig.completed`)."""
+    files = open_model_files(folder)
+    try:
+        return {n: tuple(f.info(n)[1]) for f in files for n in f.names()}
+    finally:
+        for f in files:
+            f.close()
+
+
 def load_tensors(folder: str, specs: Sequence[TensorSpec], run_dtype: torch.dtype,
                  device: torch.device) -> Dict[str, torch.Tensor]:
     files = open_model_files(folder)

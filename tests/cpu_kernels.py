@@ -257,3 +257,86 @@ class CpuKernels:
     def advance(self, row_pos, seq_start, seq_len, batch):
         for t in (row_pos, seq_start, seq_len):
             t[:batch] += 1
+
+    # ---- the kernels of the bigram embedding, the norm on a sublayer's result, gated linear attention, attention
+    # ---- through a latent and the mixture of experts ----
+    def bigram_add(self, x, table, tokens, prev, buckets, mul_prev, mul_cur, vocab, row_pos, row_seq, seq_slot, cu_rows,
+                   batch):
+        for b in range(batch):
+            r0, r1 = int(cu_rows[b]), int(cu_rows[b + 1])
+            slot = int(seq_slot[b])
+            for r in range(r0, r1):
+                tok = int(tokens[r])
+                before = int(tokens[r - 1]) if r > r0 else int(prev[slot, 0])
+                if int(row_pos[r]) == 0:
+                    x[r] += table[buckets].float()
+                elif 0 <= tok < vocab and 0 <= before < vocab:
+                    x[r] += table[(before * mul_prev + tok * mul_cur) % buckets].float()
+            prev[slot, 0] = int(tokens[r1 - 1])
+
+    def rmsnorm_residual(self, x, y, weight, eps, rounded=None):
+        yf = y.float()
+        x += yf / torch.sqrt((yf * yf).mean(-1, keepdim=True) + eps) * weight
+        if rounded is not None:
+            rounded.copy_(x.to(rounded.dtype))
+
+    def rmsnorm_cols(self, src, weight, eps, out):
+        v = src.float()
+        out.copy_((v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps) * weight).to(out.dtype))
+
+    def rotary(self, src, out, heads, size, out_head_stride, dims, interleaved, freqs, magnitude, row_pos):
+        rows = src.shape[0]
+        v = src.float().reshape(rows, heads, size).clone()
+        ang = row_pos[:rows].double()[:, None] * freqs.double()[None, :]
+        c = (torch.cos(ang) * magnitude).float()[:, None, :]
+        s = (torch.sin(ang) * magnitude).float()[:, None, :]
+        half = dims // 2
+        if interleaved:
+            a, b = v[..., 0:dims:2].clone(), v[..., 1:dims:2].clone()
+            v[..., 0:dims:2], v[..., 1:dims:2] = a * c - b * s, b * c + a * s
+        else:
+            a, b = v[..., :half].clone(), v[..., half:dims].clone()
+            v[..., :half], v[..., half:dims] = a * c - b * s, b * c + a * s
+        for h in range(heads):
+            out[:, h * out_head_stride : h * out_head_stride + size] = v[:, h].to(out.dtype)
+
+    def linear_heads(self, x, w, out, heads, out_head_stride):
+        n, k = w.shape[1], w.shape[2]
+        for h in range(heads):
+            out[:, h * out_head_stride : h * out_head_stride + n] = \
+                (x[:, h * k : (h + 1) * k].float() @ w[h].float().t()).to(out.dtype)
+
+    def gla_scan(self, q, k, v, z, bias, state, out, heads, key_dim, value_dim, q_scale, inv_tau, seq_slot, cu_rows,
+                 batch):
+        for b in range(batch):
+            r0, r1 = int(cu_rows[b]), int(cu_rows[b + 1])
+            s = state[int(seq_slot[b])]  # [heads, value_dim, key_dim]
+            for r in range(r0, r1):
+                decay = torch.exp(torch.nn.functional.logsigmoid(z[r].float() + bias) * inv_tau).reshape(heads, key_dim)
+                qr = q[r].float().reshape(heads, key_dim) * q_scale
+                kr = k[r].float().reshape(heads, key_dim)
+                vr = v[r].float().reshape(heads, value_dim)
+                s.mul_(decay[:, None, :]).add_(vr[:, :, None] * kr[:, None, :])
+                out[r] = (s * qr[:, None, :]).sum(-1).reshape(-1)
+
+    def moe_route(self, logits, route, top, renormalize=False):
+        s = torch.sigmoid(logits.float())
+        route.fill_(-1.0)
+        for r in range(s.shape[0]):
+            chosen = sorted(range(s.shape[1]), key=lambda e: (-float(s[r, e]), e))[:top]
+            total = sum(float(s[r, e]) for e in chosen) if renormalize else 1.0
+            for e in chosen:
+                route[r, e] = s[r, e] / total
+
+    def moe_glu(self, gu, route, out, experts, ff, limit, weight_input=True):
+        rows = gu.shape[0]
+        v = gu.float().reshape(rows, experts, 2, ff)
+        w = route.float()[:, :, None]
+        scale = w if weight_input else torch.ones_like(w)
+        g = torch.clamp(v[:, :, 0] * scale, max=limit)
+        u = torch.clamp(v[:, :, 1] * scale, -limit, limit)
+        y = g * torch.sigmoid(1.702 * g) * (u + 1)
+        if not weight_input:
+            y = y * w
+        y = torch.where(w >= 0, y, torch.zeros_like(y))
+        out.copy_(y.reshape(rows, experts * ff).to(out.dtype))
