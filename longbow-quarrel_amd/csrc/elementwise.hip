@@ -905,3 +905,81 @@ extern "C" int lq_rope_table(const double* freqs, const int* row_pos, float* cs,
   LQ_CHECK_LAUNCH("rope_table");
   return 0;
 }
+
+// ---------------------------------------------------------------- a second embedding table asked with a hash of two tokens
+// x[r, :] += table[row, :], row = (previous * mul_prev + token * mul_cur) mod buckets, for a sequence's first token
+// the row number `buckets`.  The token before a step's first row is the sequence's entry of `last` [slots], which
+// the workgroup of that first row reads and then overwrites with the step's last token of the sequence (nobody
+// else touches the entry).  A token that is no row of the vocabulary adds nothing.
+namespace {
+template <typename T>
+__global__ __launch_bounds__(256) void bigram_add_kernel(float* __restrict__ x, const T* __restrict__ table,
+                                                         const int* __restrict__ tokens, int* __restrict__ last,
+                                                         long long buckets, long long mul_prev, long long mul_cur,
+                                                         int vocab, int width, const int* __restrict__ row_pos,
+                                                         const int* __restrict__ row_seq, const int* __restrict__ seq_slot,
+                                                         const int* __restrict__ cu_rows) {
+  const int r = blockIdx.x;
+  const int seq = row_seq[r], first = cu_rows[seq], slot = seq_slot[seq];
+  const int tok = tokens[r];
+  const int before = r > first ? tokens[r - 1] : last[slot];
+  __syncthreads();  // every thread has read the entry before one of them writes it
+  if (r == first && threadIdx.x == 0) last[slot] = tokens[cu_rows[seq + 1] - 1];
+  long long row = -1;
+  if (row_pos[r] == 0) row = buckets;
+  else if (tok >= 0 && tok < vocab && before >= 0 && before < vocab) {
+    row = ((long long)before * mul_prev + (long long)tok * mul_cur) % buckets;
+    if (row < 0) row += buckets;
+  }
+  if (row < 0 || tok < 0 || tok >= vocab) return;
+  const T* src = table + row * width;
+  float* dst = x + (long long)r * width;
+  for (int i = threadIdx.x; i < width; i += 256) dst[i] += to_f32(src[i]);
+}
+
+// x[r, :] += y[r, :] / sqrt(mean(y[r, :]^2) + eps) * w; rounded[r, :] = x[r, :] in another dtype, where given.
+template <typename T>
+__global__ __launch_bounds__(256) void rmsnorm_residual_kernel(float* __restrict__ x, const float* __restrict__ y,
+                                                               const float* __restrict__ w, float eps,
+                                                               T* __restrict__ rounded, int width) {
+  __shared__ float red[16];
+  const long long base = (long long)blockIdx.x * width;
+  float acc = 0.f;
+  for (int i = threadIdx.x; i < width; i += 256) acc = fmaf(y[base + i], y[base + i], acc);
+  const float inv = 1.f / sqrtf(block_sum(acc, red) / (float)width + eps);
+  for (int i = threadIdx.x; i < width; i += 256) {
+    const float v = x[base + i] + y[base + i] * inv * w[i];
+    x[base + i] = v;
+    if (rounded != nullptr) rounded[base + i] = from_f32<T>(v);
+  }
+}
+}  // namespace
+
+extern "C" int lq_bigram_add(float* x, const void* table, int table_dtype, const int* tokens, int* last, long long buckets,
+                             long long mul_prev, long long mul_cur, int vocab, int rows, int width, const int* row_pos,
+                             const int* row_seq, const int* seq_slot, const int* cu_rows, hipStream_t stream) {
+  LQ_REQUIRE(rows > 0 && width > 0 && buckets > 0 && vocab > 0, "bigram_add: rows %d, width %d, buckets %lld", rows, width, buckets);
+  LQ_REQUIRE(x && table && tokens && last && row_pos && row_seq && seq_slot && cu_rows, "bigram_add: null pointer");
+  if (table_dtype == LQ_F32)
+    bigram_add_kernel<float><<<rows, 256, 0, stream>>>(x, (const float*)table, tokens, last, buckets, mul_prev, mul_cur, vocab,
+                                                       width, row_pos, row_seq, seq_slot, cu_rows);
+  else if (table_dtype == LQ_BF16)
+    bigram_add_kernel<bf16_t><<<rows, 256, 0, stream>>>(x, (const bf16_t*)table, tokens, last, buckets, mul_prev, mul_cur,
+                                                        vocab, width, row_pos, row_seq, seq_slot, cu_rows);
+  else LQ_REQUIRE(false, "bigram_add: unknown dtype %d", table_dtype);
+  LQ_CHECK_LAUNCH("bigram_add");
+  return 0;
+}
+
+extern "C" int lq_rmsnorm_residual(float* x, const float* y, const float* w, float eps, void* rounded, int rounded_dtype,
+                                   int rows, int width, hipStream_t stream) {
+  LQ_REQUIRE(rows > 0 && width > 0, "rmsnorm_residual: rows %d and width %d must be positive", rows, width);
+  LQ_REQUIRE(x && y && w, "rmsnorm_residual: null pointer");
+  if (rounded == nullptr || rounded_dtype == LQ_F32)
+    rmsnorm_residual_kernel<float><<<rows, 256, 0, stream>>>(x, y, w, eps, (float*)rounded, width);
+  else if (rounded_dtype == LQ_BF16)
+    rmsnorm_residual_kernel<bf16_t><<<rows, 256, 0, stream>>>(x, y, w, eps, (bf16_t*)rounded, width);
+  else LQ_REQUIRE(false, "rmsnorm_residual: unknown dtype %d", rounded_dtype);
+  LQ_CHECK_LAUNCH("rmsnorm_residual");
+  return 0;
+}

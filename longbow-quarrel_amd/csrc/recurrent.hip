@@ -528,6 +528,82 @@ __global__ __launch_bounds__(TH) void delta_scan_kernel(const float* __restrict_
   }
 }
 
+// Gated linear attention: S <- diag(a) S + k v^T;  o = S^T (q q_scale), with a decay for every key channel,
+// a = sigmoid(z + bias)^(inv_tau), taken as exp(inv_tau * log sigmoid(z + bias)) in 32-bit.
+// (ScanShape: groups = heads, N = key size, P = value size; the state [slots, heads, P, N].)
+// A chunk of TT tokens is staged in LDS (q, k and the decays of the head, the workgroup's slice of v), computed token
+// by token, and its results leave together.  A token's sums are a thread's own entries in ascending order, then the
+// exchange over the column's lanes: the same in every launch.
+template <int LN, int SLAB, int TH>
+__global__ __launch_bounds__(TH) void gla_scan_kernel(const float* __restrict__ q, int ldq, const float* __restrict__ k,
+                                                       int ldk, const float* __restrict__ v, int ldv,
+                                                       const float* __restrict__ z, int ldz,
+                                                       const float* __restrict__ bias, float* __restrict__ state,
+                                                       float* __restrict__ out, int ldo, ScanShape sh, float q_scale,
+                                                       float inv_tau, int TT) {
+  extern __shared__ float lds[];
+  const int heads = sh.heads, P = sh.P, N = sh.N;
+  const int b = blockIdx.x / heads, h = blockIdx.x % heads;
+  const int threads = blockDim.x, cols = threads / LN, tid = threadIdx.x;
+  const int l = tid % LN, col = tid / LN, p0 = blockIdx.y * cols, p = p0 + col;
+  const bool live = p < P;
+  constexpr int NP = LN * SLAB;  // a shared row in LDS, padded with zeros: entries past N take part as zeros
+  float* qs = lds;               // [TT][NP]
+  float* ks = qs + TT * NP;      // [TT][NP]
+  float* as = ks + TT * NP;      // [TT][NP]
+  float* vs = as + TT * NP;      // [TT][cols]
+  float* os = vs + TT * cols;    // [TT][cols]
+  const long long r0 = sh.cu_rows[b], r1 = sh.cu_rows[b + 1];
+  float* sp = state + (((long long)sh.seq_slot[b] * heads + h) * P + (live ? p : 0)) * N;
+  float S[SLAB];
+#pragma unroll
+  for (int i = 0; i < SLAB; ++i) {
+    const int n = i * LN + l;
+    S[i] = (live && n < N) ? sp[n] : 0.f;
+  }
+  for (int e = tid; e < 3 * TT * NP; e += threads) lds[e] = 0.f;
+  __syncthreads();
+  for (long long c0 = r0; c0 < r1; c0 += TT) {
+    const int nt = (int)min((long long)TT, r1 - c0);
+    for (int e = tid; e < nt * N; e += threads) {
+      const int t = e / N, n = e - t * N;
+      const long long r = c0 + t;
+      qs[t * NP + n] = q[r * ldq + h * N + n] * q_scale;
+      ks[t * NP + n] = k[r * ldk + h * N + n];
+      as[t * NP + n] = expf(-softplus_f(-(z[r * ldz + h * N + n] + bias[h * N + n])) * inv_tau);
+    }
+    for (int e = tid; e < nt * cols; e += threads) {
+      const int t = e / cols, c = e - t * cols;
+      vs[e] = p0 + c < P ? v[(c0 + t) * ldv + h * P + p0 + c] : 0.f;
+    }
+    __syncthreads();
+    for (int t = 0; t < nt; ++t) {
+      const float vv = vs[t * cols + col];
+      float acc = 0.f;
+#pragma unroll
+      for (int i = 0; i < SLAB; ++i) {
+        const int n = t * NP + i * LN + l;
+        S[i] = fmaf(ks[n], vv, as[n] * S[i]);
+        acc = fmaf(S[i], qs[n], acc);
+      }
+      acc = group_sum<LN>(acc);
+      if (l == 0) os[t * cols + col] = acc;
+    }
+    __syncthreads();
+    for (int e = tid; e < nt * cols; e += threads) {
+      const int t = e / cols, c = e - t * cols;
+      if (p0 + c < P) out[(c0 + t) * ldo + h * P + p0 + c] = os[e];
+    }
+  }
+  if (live) {
+#pragma unroll
+    for (int i = 0; i < SLAB; ++i) {
+      const int n = i * LN + l;
+      if (n < N) sp[n] = S[i];
+    }
+  }
+}
+
 // ---------------------------------------------------------------- norms after the scans
 // One workgroup a (row, group of `group` columns).  gate_first: v = y silu(z), out = v / rms(v) w;
 // else: out = y / rms(y) w silu(z).  w has `wlen` entries and repeats (one weight for all groups, or one a column).
@@ -826,5 +902,32 @@ extern "C" int lq_rmsnorm_mean(const float* stack, int n_in, const float* w0, co
   LQ_REQUIRE(stack && out, "rmsnorm_mean: null pointer");
   rmsnorm_mean_kernel<<<rows, width >= 4096 ? 1024 : width >= 1024 ? 256 : 64, 0, stream>>>(in, n_in, eps, out, width);
   LQ_CHECK_LAUNCH("rmsnorm_mean");
+  return 0;
+}
+
+// q, k and z [rows, heads * Dk] (z: the decay's logits, before bias), v [rows, heads * P], bias [heads * Dk], state
+// [slots, heads, P, Dk], out [rows, heads * P]
+extern "C" int lq_gla_scan(const float* q, int ldq, const float* k, int ldk, const float* v, int ldv, const float* z, int ldz,
+                           const float* bias, float* state, float* out, int ldo, int heads, int Dk, int P, float q_scale,
+                           float inv_tau, const int* seq_slot, const int* cu_rows, int batch, hipStream_t stream) {
+  LQ_REQUIRE(heads > 0 && Dk > 0 && P > 0 && batch > 0, "gla_scan: bad sizes");
+  LQ_REQUIRE(ldq >= heads * Dk && ldk >= heads * Dk && ldz >= heads * Dk && ldv >= heads * P && ldo >= heads * P,
+             "gla_scan: a row stride is smaller than its row");
+  LQ_REQUIRE(q && k && v && z && bias && state && out && seq_slot && cu_rows, "gla_scan: null pointer");
+  ScanLaunch cfg;
+  LQ_REQUIRE(scan_launch(Dk, P, (long long)batch * heads, cfg), "gla_scan: key size %d is too large", Dk);
+  const int np = cfg.ln * cfg.slab;
+  int tt = 8;
+  while (tt > 1 && (size_t)tt * (3 * np + 2 * cfg.cols) * sizeof(float) > 64 * 1024) tt >>= 1;
+  const size_t lds = (size_t)tt * (3 * np + 2 * cfg.cols) * sizeof(float);
+  LQ_REQUIRE(lds <= 64 * 1024, "gla_scan: key size %d is too large", Dk);
+  dim3 grid((unsigned)(batch * heads), lq_ceil_div(P, cfg.cols));
+  ScanShape sh = {heads, heads, P, Dk, seq_slot, cu_rows};
+#define LQ_GLA(LN, SL, TH)                                                                                            \
+  gla_scan_kernel<LN, SL, TH><<<grid, cfg.threads, lds, stream>>>(q, ldq, k, ldk, v, ldv, z, ldz, bias, state, out, ldo, \
+                                                                  sh, q_scale, inv_tau, tt)
+  LQ_SCAN_LANES(LQ_GLA)
+#undef LQ_GLA
+  LQ_CHECK_LAUNCH("gla_scan");
   return 0;
 }

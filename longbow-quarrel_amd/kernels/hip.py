@@ -20,7 +20,7 @@ from .. import build as _build
 from .dry import query
 
 F32, BF16 = 0, 1
-ABI_VERSION = 6  # lq_abi_version() of the library these wrappers were written for
+ABI_VERSION = 7  # lq_abi_version() of the library these wrappers were written for
 _DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
 
 
@@ -897,6 +897,141 @@ class HipKernels:
         ws = [_ptr(w) for w in weights] + [c_void_p(0)] * (4 - n)
         self._check(self.lib.lq_rmsnorm_mean(_ptr(stack), c_int(n), *ws, c_float(eps), _ptr(out), c_int(rows),
                                              c_int(width), self.stream))
+
+    # ------------------------------------------------------------------ bigram embedding, norm on a sublayer's result,
+    # ------------------------------------------------------------------ gated linear attention, latent attention, experts
+    def bigram_add(self, x: torch.Tensor, table: torch.Tensor, tokens: torch.Tensor, last: torch.Tensor, buckets: int,
+                   mul_prev: int, mul_cur: int, vocab: int, row_pos: torch.Tensor, row_seq: torch.Tensor,
+                   seq_slot: torch.Tensor, cu_rows: torch.Tensor, batch: int) -> None:
+        """x[r] += table[(previous * mul_prev + token * mul_cur) mod buckets] (row `buckets` for a sequence's first
+        token); the token before a step's first row comes from last[slot], which then takes the step's last token."""
+        self._dev(x, table, tokens, last, row_pos, row_seq, seq_slot, cu_rows)
+        rows, width = x.shape
+        if x.dtype != torch.float32 or not x.is_contiguous() or table.dim() != 2 or not table.is_contiguous() \
+                or tuple(table.shape) != (buckets + 1, width):
+            raise KernelLibraryError(f"bigram_add: x dense float32 [rows, width], the table dense [{buckets + 1}, width]")
+        if last.dtype != torch.int32 or not last.is_contiguous() or last.numel() != last.shape[0]:
+            raise KernelLibraryError("bigram_add: the last tokens are a dense int32 entry a slot")
+        for t, what, n in ((tokens, "tokens", rows), (row_pos, "row_pos", rows), (row_seq, "row_seq", rows),
+                           (seq_slot, "seq_slot", batch), (cu_rows, "cu_rows", batch + 1)):
+            self._i32(t, what, n)
+        self._check(self.lib.lq_bigram_add(_ptr(x), _ptr(table), c_int(_code(table)), _ptr(tokens), _ptr(last),
+                                           c_longlong(buckets), c_longlong(mul_prev), c_longlong(mul_cur), c_int(vocab),
+                                           c_int(rows), c_int(width), _ptr(row_pos), _ptr(row_seq), _ptr(seq_slot),
+                                           _ptr(cu_rows), self.stream))
+
+    def rmsnorm_residual(self, x: torch.Tensor, y: torch.Tensor, weight: torch.Tensor, eps: float,
+                         rounded: Optional[torch.Tensor] = None) -> None:
+        """x += y / sqrt(mean(y^2) + eps) * weight, row by row (x and y float32); `rounded`, where given, takes the
+        new x in its own dtype."""
+        self._dev(x, y, weight, rounded)
+        rows, width = x.shape
+        if x.dtype != torch.float32 or y.dtype != torch.float32 or tuple(y.shape) != (rows, width) \
+                or not x.is_contiguous() or not y.is_contiguous():
+            raise KernelLibraryError("rmsnorm_residual: x and y must be dense float32 of one shape")
+        self._f32(weight, "rmsnorm_residual: weight", width)
+        if rounded is not None and (tuple(rounded.shape) != (rows, width) or not rounded.is_contiguous()):
+            raise KernelLibraryError("rmsnorm_residual: rounded must be dense and shaped like x")
+        self._check(self.lib.lq_rmsnorm_residual(_ptr(x), _ptr(y), _ptr(weight), c_float(eps), _ptr(rounded),
+                                                 c_int(_code(rounded) if rounded is not None else 0), c_int(rows),
+                                                 c_int(width), self.stream))
+
+    def rmsnorm_cols(self, src: torch.Tensor, weight: torch.Tensor, eps: float, out: torch.Tensor) -> None:
+        """out = src / sqrt(mean(src^2) + eps) * weight, row by row; src float32 [rows, n] and out [rows, n] may
+        each be a run of columns of a wider row."""
+        rows, n, lds = self._mat(src, "rmsnorm_cols: src")
+        ro, no, ldo = self._mat(out, "rmsnorm_cols: out")
+        if src.dtype != torch.float32 or (ro, no) != (rows, n):
+            raise KernelLibraryError("rmsnorm_cols: src float32 [rows, n], out [rows, n]")
+        self._f32(weight, "rmsnorm_cols: weight", n)
+        self._check(self.lib.lq_rmsnorm_cols(_ptr(src), c_int(lds), _ptr(weight), c_float(eps), _ptr(out),
+                                             c_int(_code(out)), c_int(ldo), c_int(rows), c_int(n), self.stream))
+
+    def rotary(self, src: torch.Tensor, out: torch.Tensor, heads: int, size: int, out_head_stride: int, dims: int,
+               interleaved: bool, freqs: torch.Tensor, magnitude: float, row_pos: torch.Tensor) -> None:
+        """Head h of row r: src[r, h size .. + size) (float32) goes to out[r, h out_head_stride .. + size), its first
+        `dims` entries rotated by row_pos[r] * freqs (float64 [dims / 2]) in half-split pairs (j, j + dims / 2) or
+        interleaved pairs (2 j, 2 j + 1), cos and sin times `magnitude`.  `out` starts at the first entry written
+        and may be a run of columns of a wider row."""
+        rows, ns, lds = self._mat(src, "rotary: src")
+        ro, no, ldo = self._mat(out, "rotary: out")
+        self._i32(row_pos, "row_pos", rows)
+        if src.dtype != torch.float32 or ns != heads * size or ro != rows or no < (heads - 1) * out_head_stride + size:
+            raise KernelLibraryError("rotary: src float32 [rows, heads * size], out with room for every head's vector")
+        if freqs.dtype != torch.float64 or not freqs.is_cuda or not freqs.is_contiguous() or freqs.numel() != dims // 2:
+            raise KernelLibraryError(f"rotary: {dims // 2} float64 frequencies on the GPU")
+        self._check(self.lib.lq_rotary(_ptr(src), c_int(lds), _ptr(out), c_int(_code(out)), c_int(ldo), c_int(rows),
+                                       c_int(heads), c_int(size), c_int(out_head_stride), c_int(dims),
+                                       c_int(1 if interleaved else 0), _ptr(freqs), c_float(magnitude), _ptr(row_pos),
+                                       self.stream))
+
+    def linear_heads(self, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, heads: int, out_head_stride: int) -> None:
+        """A product a head: out[r, h out_head_stride .. + N) = x[r, h K .. + K) . w[h]^T with w [heads, N, K]."""
+        rows, kx, ldx = self._mat(x, "linear_heads: x")
+        ro, no, ldc = self._mat(out, "linear_heads: out")
+        if w.dim() != 3 or not w.is_contiguous() or not w.is_cuda or w.shape[0] != heads or kx != heads * w.shape[2] \
+                or ro != rows or no < (heads - 1) * out_head_stride + w.shape[1] or out_head_stride < w.shape[1] \
+                or x.dtype != w.dtype:
+            raise KernelLibraryError(f"linear_heads: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not fit")
+        n, k = int(w.shape[1]), int(w.shape[2])
+        xe, we, oe = x.element_size(), w.element_size(), out.element_size()
+        cx, co = _code(x), _code(out)
+        generic = 1 if self.force_generic else 0
+        for h in range(heads):
+            rc = self.lib.lq_linear(x.data_ptr() + h * k * xe, w.data_ptr() + h * n * k * we,
+                                    out.data_ptr() + h * out_head_stride * oe, cx, co, rows, n, k, ldx, k, ldc, 1, 0,
+                                    generic, 0, self.stream)
+            if rc:
+                self._check(rc)
+
+    def gla_scan(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z: torch.Tensor, bias: torch.Tensor,
+                 state: torch.Tensor, out: torch.Tensor, heads: int, key_dim: int, value_dim: int, q_scale: float,
+                 inv_tau: float, seq_slot: torch.Tensor, cu_rows: torch.Tensor, batch: int) -> None:
+        """Gated linear attention along every sequence of the step, token by token: with the decay a =
+        sigmoid(z + bias)^inv_tau for every key channel, S <- diag(a) S + k v^T and out = S^T (q q_scale) per head;
+        state [slots, heads, value_dim, key_dim] is read and left at the step's end.  All float32."""
+        rows = q.shape[0]
+        for t, what, cols in ((q, "q", heads * key_dim), (k, "k", heads * key_dim), (z, "z", heads * key_dim),
+                              (v, "v", heads * value_dim), (out, "out", heads * value_dim)):
+            self._f32(t, "gla_scan: " + what)
+            if self._mat(t, "gla_scan: " + what)[:2] != (rows, cols):
+                raise KernelLibraryError(f"gla_scan: {what} must be [{rows}, {cols}], found {tuple(t.shape)}")
+        self._f32(bias, "gla_scan: bias", heads * key_dim)
+        self._f32(state, "gla_scan: state")
+        if state.dim() != 4 or tuple(state.shape[1:]) != (heads, value_dim, key_dim) or not state.is_contiguous():
+            raise KernelLibraryError("gla_scan: state must be dense [slots, heads, value_dim, key_dim]")
+        self._i32(seq_slot, "seq_slot", batch)
+        self._i32(cu_rows, "cu_rows", batch + 1)
+        ld = self._rows2d
+        self._check(self.lib.lq_gla_scan(_ptr(q), c_int(ld(q, "q")), _ptr(k), c_int(ld(k, "k")), _ptr(v),
+                                         c_int(ld(v, "v")), _ptr(z), c_int(ld(z, "z")), _ptr(bias), _ptr(state), _ptr(out),
+                                         c_int(ld(out, "out")), c_int(heads), c_int(key_dim), c_int(value_dim),
+                                         c_float(q_scale), c_float(inv_tau), _ptr(seq_slot), _ptr(cu_rows), c_int(batch),
+                                         self.stream))
+
+    def moe_route(self, logits: torch.Tensor, route: torch.Tensor, top: int, renormalize: bool = False) -> None:
+        """route[r, e] = sigmoid(logits[r, e]) for the `top` experts with the largest scores (the lower index on a
+        tie; divided by the chosen scores' sum with `renormalize`), -1 for the others.  float32."""
+        rows, experts, ldz = self._mat(logits, "moe_route: logits")
+        self._f32(logits, "moe_route: logits")
+        self._f32(route, "moe_route: route", rows * experts)
+        self._check(self.lib.lq_moe_route(_ptr(logits), c_int(ldz), _ptr(route), c_int(rows), c_int(experts), c_int(top),
+                                          c_int(1 if renormalize else 0), self.stream))
+
+    def moe_glu(self, gu: torch.Tensor, route: torch.Tensor, out: torch.Tensor, experts: int, ff: int, limit: float,
+                weight_input: bool = True) -> None:
+        """gu [rows, experts * 2 ff] float32 (every expert's gate then up), route [rows, experts]; out [rows,
+        experts * ff]: for a chosen expert with weight w, g = min(w gate, limit), u = clamp(w up, -limit, limit),
+        y = g sigmoid(1.702 g) (u + 1) (with `weight_input` false w multiplies y instead); 0 for the others."""
+        rows, ng, ldg = self._mat(gu, "moe_glu: gu")
+        ro, no, ldo = self._mat(out, "moe_glu: out")
+        self._f32(gu, "moe_glu: gu")
+        self._f32(route, "moe_glu: route", rows * experts)
+        if ng != experts * 2 * ff or (ro, no) != (rows, experts * ff):
+            raise KernelLibraryError("moe_glu: gu [rows, experts * 2 ff] and out [rows, experts * ff]")
+        self._check(self.lib.lq_moe_glu(_ptr(gu), c_longlong(ldg), _ptr(route), _ptr(out), c_int(_code(out)),
+                                        c_longlong(ldo), c_int(rows), c_int(experts), c_int(ff), c_float(limit),
+                                        c_int(1 if weight_input else 0), self.stream))
 
     # ------------------------------------------------------------------ sampling
     @property
