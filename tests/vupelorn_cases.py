@@ -1,0 +1,177 @@
+"""Configurations, weights and the engine-beside-plain case for the Vupelorn tests, shared by the CPU tests (the
+engine's own code over the torch stand-in for the kernels) and the GPU tests (the same over the HIP kernels).
+Every comparison is against `plain_vupelorn`, run over whole sequences in float64.  The scenarios (cuttings,
+batches, reuse of slots, long decoding, greedy tokens) are those of `vafodra_cases`, which ask nothing of a case
+but its engine, its vocabulary and the plain logits."""
+from __future__ import annotations
+
+import copy
+from typing import Dict, List
+
+import torch
+
+import longbow_quarrel_amd as lq
+import plain_vupelorn as pv
+from vafodra_cases import (err, greedy, long_decoding, portions, slots_and_blocks_used_again, tokens,  # noqa: F401
+                           unequal_batches, whole_and_token_by_token, write_folder)
+from longbow_quarrel_amd.engine import StepEntry
+
+
+def _moe(experts, top, ff, limit):
+    return {"kind": "moe", "expert": {"ff": ff, "limit": limit}, "router": {"experts": experts, "top": top}}
+
+
+def _gla(heads, dim, vdim, tau, rank, mlp=None):
+    return {"type": "gla", "mixer": {"heads": heads, "dim": dim, "vdim": vdim, "tau": tau, "decay_rank": rank}, "mlp": mlp}
+
+
+def _latent(kind, heads, dim, rot_dim, vdim, kv_rank, q_rank, scale, base, mlp=None, rot_dims=None, scaling=None,
+            kv_from=None):
+    rot = {"base": base, "dims": rot_dim if rot_dims is None else rot_dims}
+    if scaling is not None:
+        rot["scaling"] = scaling
+    m = {"heads": heads, "dim": dim, "rot_dim": rot_dim, "vdim": vdim, "kv_rank": kv_rank, "q_rank": q_rank,
+         "scale": scale, "rot": rot}
+    if kv_from is not None:
+        m["kv_from"] = kv_from
+    return {"type": kind, "mixer": m, "mlp": mlp}
+
+
+def _config(vocab, width, eps, layers, bigram=None):
+    d = {"architecture": "Vupelorn", "layers": layers, "norm": {"eps": eps}, "vocab": vocab, "width": width}
+    if bigram is not None:
+        d["embedding"] = {"bigram": dict(zip(("buckets", "mul_prev", "mul_cur"), bigram))}
+    return d
+
+
+_YARN = {"factor": 8.0, "original": 40, "fast": 16.0, "slow": 2.0}
+# A: every kind of layer; YaRN whose blend lies inside the pairs; a layer without feed-forward; a layer that reads
+# another's latent with other head counts and sizes of its own; all experts chosen in one layer, one in another;
+# tau 1; a bigram table
+CFG_A = _config(211, 96, 1e-6, [
+    _latent("latent_attention", 3, 16, 16, 32, 48, 40, 0.2, 5000.0, _moe(5, 2, 24, 1.5), scaling=_YARN),
+    _gla(2, 40, 24, 8.0, 6),
+    _latent("latent_attention_2", 4, 32, 8, 16, 32, 24, 0.15, 10000.0, _moe(3, 1, 40, 3.0)),
+    _latent("latent_attention_2", 2, 16, 8, 48, 32, 56, 0.3, 10000.0, _moe(4, 4, 16, 0.5), kv_from=2),
+    _gla(3, 8, 8, 1.0, 2, _moe(2, 1, 32, 2.0)),
+], bigram=(97, 13, 5))
+# B: sizes that are multiples of nothing (the kernels' size-agnostic ways), no bigram table, a rotation of fewer
+# entries than the rotated part holds, one head, a gated-linear-attention layer first and a shared latent two
+# layers back
+CFG_B = _config(131, 50, 1e-5, [
+    _gla(1, 17, 9, 3.5, 3, _moe(2, 1, 9, 1.0)),
+    _latent("latent_attention_2", 5, 10, 6, 7, 13, 11, 0.25, 300.0, None, rot_dims=4),
+    _latent("latent_attention", 1, 24, 10, 12, 20, 18, 0.2, 1000.0, _moe(3, 2, 10, 2.5),
+            scaling={"factor": 2.0, "original": 16, "fast": 4.0, "slow": 1.0}),
+    _latent("latent_attention_2", 2, 6, 6, 10, 13, 9, 0.4, 300.0, None, rot_dims=4, kv_from=1),
+], bigram=None)
+# C: head sizes, ranks and widths of the kind that the fast kernels are made for
+CFG_C = _config(1000, 256, 1e-5, [
+    _latent("latent_attention", 4, 64, 32, 64, 96, 128, 0.1, 10000.0, _moe(4, 2, 128, 7.0),
+            scaling={"factor": 4.0, "original": 128, "fast": 32.0, "slow": 1.0}),
+    _gla(4, 64, 64, 16.0, 16, _moe(8, 2, 64, 7.0)),
+    _latent("latent_attention_2", 8, 32, 16, 32, 48, 64, 0.14, 10000.0, _moe(4, 1, 128, 7.0)),
+    _latent("latent_attention_2", 16, 16, 16, 16, 48, 64, 0.2, 10000.0, None, kv_from=2),
+], bigram=(509, 3, 11))
+# one mechanism a model: what fails here names its mechanism
+CFG_GLA = _config(60, 48, 1e-6, [_gla(3, 16, 8, 4.0, 4)], bigram=None)
+CFG_LATENT = _config(60, 48, 1e-6, [
+    _latent("latent_attention", 2, 16, 8, 24, 16, 12, 0.25, 100.0, scaling={"factor": 3.0, "original": 20, "fast": 8.0, "slow": 1.0})])
+CFG_LATENT2 = _config(60, 48, 1e-6, [
+    _latent("latent_attention_2", 2, 16, 8, 24, 16, 12, 0.25, 100.0),
+    _latent("latent_attention_2", 3, 8, 8, 16, 16, 20, 0.3, 100.0, kv_from=0)])
+CFG_MOE = _config(60, 48, 1e-6, [_gla(1, 8, 8, 2.0, 2, _moe(6, 3, 20, 1.0))], bigram=None)
+CFG_BIGRAM = _config(60, 48, 1e-6, [_gla(1, 8, 8, 2.0, 2)], bigram=(7, 1000003, 999983))
+CONFIGS = {"a": CFG_A, "b": CFG_B, "c": CFG_C, "gla": CFG_GLA, "latent": CFG_LATENT, "latent2": CFG_LATENT2,
+           "moe": CFG_MOE, "bigram": CFG_BIGRAM}
+
+
+def make_weights(cfg: dict, seed: int, sharp: float = 1.0, memory: float = 0.0) -> Dict[str, torch.Tensor]:
+    """Random weights whose values bfloat16 holds exactly (both run dtypes then see the same model), with spreads
+    that make every constant matter.  `sharp` scales the queries' and the latents' projections so that attention
+    is peaked (a far key can then carry a row's result); `memory` is added to the decays' biases, so that a gated
+    linear attention state forgets slowly and old tokens stay in it."""
+    config = lq.VupelornConfig.from_dict(cfg)
+    from longbow_quarrel_amd.model import DecoderModel
+    from longbow_quarrel_amd.registry import spec_from_config
+
+    g = torch.Generator().manual_seed(seed)
+    out = {}
+    for s in DecoderModel(spec_from_config(config)).tensor_specs():
+        n, shape = s.name, tuple(s.shape)
+        leaf = n.split(".")[-1]
+        normal = lambda std, mean=0.0: torch.empty(shape).normal_(mean, std, generator=g)
+        if n in ("embed", "bigram"):
+            t = normal(0.5)
+        elif leaf in ("norm", "norm1", "norm2") or n == "final.norm":
+            t = normal(0.3, 1.0)
+        elif n.endswith("a2.b"):
+            t = normal(1.0, 1.0 + memory)
+        elif leaf == "router":  # (scores well inside (0, 1): two that both round to 1 in 32-bit would be a tie there)
+            t = normal(0.5 / (shape[-1] ** 0.5))
+        else:
+            t = normal(1.0 / (shape[-1] ** 0.5))
+            if leaf in ("uq", "dkv"):
+                t = t * sharp
+        out[n] = t.to(torch.bfloat16).float()
+    return out
+
+
+def assert_close_bf16(got: torch.Tensor, want: torch.Tensor, typical: float = 2e-2, most: float = 6e-2) -> None:
+    """A bfloat16 run against the plain implementation that rounds where such a run does.  Rounding moves a
+    router's score by a few thousandths, so now and then a token's close call between two experts falls the other
+    way and that row differs by much more than rounding: the rows' typical error and the share of rows beyond a
+    larger limit are bounded, not the worst row."""
+    got, want = got.detach().double().cpu(), want.detach().double().cpu()
+    assert got.shape == want.shape
+    rows = (got - want).abs().max(-1).values / want.abs().max()
+    assert float(rows.median()) < typical, float(rows.median())
+    assert float((rows > most).double().mean()) <= 0.1, sorted(rows.tolist())[-8:]
+
+
+class Case:
+    """An engine (made by `load`, which the CPU and the GPU tests bring) beside the plain implementation."""
+
+    def __init__(self, tmp_path, name: str, load, dtype: str = "float32", seed: int = 3, sharp: float = 1.0,
+                 memory: float = 0.0, max_tokens: int = 2048, rounding: bool = False) -> None:
+        self.cfg = copy.deepcopy(CONFIGS[name])
+        self.weights = make_weights(self.cfg, seed, sharp, memory)
+        self.folder = write_folder(tmp_path, self.cfg, self.weights, f"{name}_{seed}_{sharp}_{memory}")
+        self.eng = load(self.folder, dtype, max_tokens)
+        self.vocab = self.cfg["vocab"]
+        self.rounding = rounding
+        self._want = {}
+
+    def want(self, toks: List[int]) -> torch.Tensor:
+        key = tuple(toks)
+        if key not in self._want:
+            self._want[key] = pv.forward(self.cfg, self.weights, toks, rounding=self.rounding)
+        return self._want[key]
+
+    def run_cut(self, toks: List[int], cuts: List[int]) -> torch.Tensor:
+        """The sequence in portions of the sizes `cuts` (the rest token by token), all logits."""
+        eng = self.eng
+        s = eng.new_sequence()
+        got, at = [], 0
+        sizes = list(cuts)
+        while at < len(toks):
+            n = min(sizes.pop(0) if sizes else 1, len(toks) - at)
+            got.append(eng.step([StepEntry(s, toks[at : at + n], range(n))]).clone())
+            at += n
+        eng.release(s)
+        return torch.cat(got)
+
+    def layers(self, toks: List[int]):
+        """The residual stream after every layer, from the engine's observer and from the plain implementation."""
+        got = []
+        s = self.eng.new_sequence()
+        self.eng.step([StepEntry(s, toks, [])],
+                      observe=lambda name, x, pending: got.append(x.float().cpu().clone()) if name != "embed" else None)
+        self.eng.release(s)
+        want = []
+        pv.forward(self.cfg, self.weights, toks, rounding=self.rounding, layers_out=want)
+        return got, want
+
+    def assert_idle(self) -> None:
+        c = self.eng.cache
+        assert c.slots.taken_count == 0 and all(g.blocks.taken_count == 0 for g in c.kv_groups)
