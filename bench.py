@@ -28,6 +28,10 @@ layer sizes of a real model, beside the Llama shape of the same width, depth, fe
 of `--design-widths` a prefill of `--prefill-tokens` tokens and decoding at `--batch` from `--prompt-len`-token
 prompts (captured steps), then device time by operation for both (events around every kernel call).  One JSON line;
 the default run is not changed by it.
+`--design vupelorn`: the same for the design of gated linear attention, attention through a cached latent and a
+mixture of experts (per four layers one gated-linear-attention layer, one latent-attention layer with YaRN, one with
+interleaved pairs and one that reads that layer's latent; 8 experts of which a token uses 2, their inner sizes
+such that a token's two experts together are as wide as the Llama shape's feed-forward).
 """
 from __future__ import annotations
 
@@ -100,6 +104,32 @@ def vafodra_config(width: int, layers: int, vocab: int) -> dict:
             "residual_mult": 0.5, "vocab": vocab, "width": width}
 
 
+def vupelorn_config(width: int, layers: int, vocab: int) -> dict:
+    """Layer sizes of a real model for the design: heads of 128 unrotated and 64 rotated entries over a latent of
+    192 (a cached row of 256), queries through a latent of 3/8 of the width; gated linear attention with keys of
+    128 and values of 256 a head; 8 experts, 2 a token, each 1.75 times the width (the two together: the Llama
+    shape's 3.5 times)."""
+    heads = width // 128
+    rot = {"base": 10000.0, "dims": 64}
+    latent = {"heads": heads, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 192, "q_rank": width * 3 // 8,
+              "scale": 192 ** -0.5, "rot": rot}
+    yarn = dict(latent, rot=dict(rot, scaling={"factor": 4.0, "original": 4096, "fast": 32.0, "slow": 1.0}))
+    gla = {"heads": width // 256, "dim": 128, "vdim": 256, "tau": 16.0, "decay_rank": 16}
+    mlp = {"kind": "moe", "expert": {"ff": width * 7 // 4, "limit": 7.0}, "router": {"experts": 8, "top": 2}}
+    made = []
+    for i in range(layers):
+        if i % 4 == 0:
+            made.append({"type": "gla", "mixer": gla, "mlp": mlp})
+        elif i % 4 == 1:
+            made.append({"type": "latent_attention", "mixer": yarn, "mlp": mlp})
+        elif i % 4 == 2:
+            made.append({"type": "latent_attention_2", "mixer": latent, "mlp": mlp})
+        else:
+            made.append({"type": "latent_attention_2", "mixer": dict(latent, kv_from=i - 1), "mlp": mlp})
+    return {"architecture": "Vupelorn", "embedding": {"bigram": {"buckets": 65521, "mul_prev": 31, "mul_cur": 7}},
+            "layers": made, "norm": {"eps": 1e-6}, "vocab": vocab, "width": width}
+
+
 def design_run(args) -> int:
     import torch
 
@@ -114,8 +144,9 @@ def design_run(args) -> int:
     for width in [int(w) for w in args.design_widths.split(",")]:
         llama = dict(CONFIG_8B, hidden_size=width, intermediate_size=width * 7 // 2, num_hidden_layers=layers,
                      num_attention_heads=width // 128, num_key_value_heads=max(1, width // 512), vocab_size=vocab)
-        for name, config in (("vafodra", lq.VafodraConfig.from_dict(vafodra_config(width, layers, vocab))),
-                             ("llama", lq.LlamaConfig.from_dict(llama))):
+        design = lq.VafodraConfig.from_dict(vafodra_config(width, layers, vocab)) if args.design == "vafodra" \
+            else lq.VupelornConfig.from_dict(vupelorn_config(width, layers, vocab))
+        for name, config in ((args.design, design), ("llama", lq.LlamaConfig.from_dict(llama))):
             engine = lq.random_engine(config, seed=0, dtype=args.dtype, max_tokens=batch * 4096 + n_prefill + 64,
                                       max_slots=batch + 1, max_sequence_tokens=max(4096, n_prefill))
             prompt = lambda n: torch.randint(0, vocab, (n,), generator=gen).tolist()
@@ -173,7 +204,8 @@ def design_run(args) -> int:
             results.append(line)
             del engine, backend, timed
             torch.cuda.empty_cache()
-    print(json.dumps({"metric": "prefill and decode tok/s of the Vafodra design beside the Llama shape of equal size",
+    print(json.dumps({"metric": f"prefill and decode tok/s of the {args.design.capitalize()} design beside the Llama shape "
+                                "of equal size",
                       "dtype": args.dtype, "data": "synthetic: random weights from a seed, uniform random token ids",
                       "n_gpus": 1, "steps": args.steps, "warmup": args.warmup, "results": results}), flush=True)
     return 0
@@ -203,7 +235,7 @@ def main() -> int:
                     help="float32: the true 32-bit path (use --layers with the larger shapes)")
     ap.add_argument("--context", type=int, default=0,
                     help="tokens a sequence may hold (default: the shape's 8192); for decoding over longer prompts")
-    ap.add_argument("--design", choices=["vafodra"], default=None,
+    ap.add_argument("--design", choices=["vafodra", "vupelorn"], default=None,
                     help="measure this design beside the Llama shape of equal size instead of the default workload")
     ap.add_argument("--design-widths", default="2048,4096", help="model widths of --design, with commas between them")
     args = ap.parse_args()

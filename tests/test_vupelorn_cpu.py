@@ -290,4 +290,4 @@ def test_greedy_generation_through_the_generation_loop(cases):
 def test_bfloat16_run_rounds_where_the_plain_implementation_does(tmp_path_factory):
     case = uc.Case(tmp_path_factory.mktemp("vupelorn16"), "a", load, dtype="bfloat16", rounding=True)
     t = uc.tokens(80, case.vocab, 3)
-    uc.assert_close_bf16(case.run_cut(t, [50, 2]), case.want(t))
+    uc.assert_close_bf16(case.run_cut(t, [50, 2]), case.want(t), case.noise(t))

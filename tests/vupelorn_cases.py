@@ -117,15 +117,21 @@ def make_weights(cfg: dict, seed: int, sharp: float = 1.0, memory: float = 0.0) 
     return out
 
 
-def assert_close_bf16(got: torch.Tensor, want: torch.Tensor, typical: float = 2e-2, most: float = 6e-2) -> None:
+def assert_close_bf16(got: torch.Tensor, want: torch.Tensor, noise: float, most: float = 0.25) -> None:
     """A bfloat16 run against the plain implementation that rounds where such a run does.  Rounding moves a
     router's score by a few thousandths, so now and then a token's close call between two experts falls the other
-    way and that row differs by much more than rounding: the rows' typical error and the share of rows beyond a
-    larger limit are bounded, not the worst row."""
+    way; that row then differs by much more than rounding, and so, less, do the rows after it, which read it
+    through the recurrent states and the cached latents.  (Measured on these configurations over 150 tokens: the
+    plain implementation with against without rounding has a median row error of 0.003 to 0.022 and single rows up
+    to 0.42; the engine over the torch stand-in and over the HIP kernels differ from it alike, median 0.018, single
+    rows up to 0.75.)  So the rows' typical error is held against three times what rounding alone does to the
+    plain implementation on the same tokens (`noise`, from `Case.noise`), and the share of rows beyond a larger
+    limit is bounded, not the worst row; the sharp comparisons are the float32 ones, through the same kernels'
+    32-bit forms."""
     got, want = got.detach().double().cpu(), want.detach().double().cpu()
     assert got.shape == want.shape
     rows = (got - want).abs().max(-1).values / want.abs().max()
-    assert float(rows.median()) < typical, float(rows.median())
+    assert float(rows.median()) < 3 * noise, (float(rows.median()), noise)
     assert float((rows > most).double().mean()) <= 0.1, sorted(rows.tolist())[-8:]
 
 
@@ -147,6 +153,13 @@ class Case:
         if key not in self._want:
             self._want[key] = pv.forward(self.cfg, self.weights, toks, rounding=self.rounding)
         return self._want[key]
+
+    def noise(self, toks: List[int]) -> float:
+        """What rounding alone does on these tokens: the median over the rows of the largest difference (over the
+        largest logit) between the plain implementation with and without rounding."""
+        a = pv.forward(self.cfg, self.weights, toks, rounding=True)
+        b = pv.forward(self.cfg, self.weights, toks, rounding=False)
+        return float(((a - b).abs().max(-1).values / b.abs().max()).median())
 
     def run_cut(self, toks: List[int], cuts: List[int]) -> torch.Tensor:
         """The sequence in portions of the sizes `cuts` (the rest token by token), all logits."""
