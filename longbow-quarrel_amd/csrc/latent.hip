@@ -62,6 +62,48 @@ __global__ __launch_bounds__(128) void rotary_kernel(const float* __restrict__ s
   }
 }
 
+// A product a head: out[r, h ohs + n] = sum_k x[r, h K + k] w[h, n, k], bfloat16 operands on
+// v_mfma_f32_16x16x16_bf16 (exact products, 32-bit sums).  A workgroup of four wavefronts takes 64 rows by 64
+// columns of one head; a wavefront 16 rows by the 64 columns, its operands straight from memory (a head's weight
+// is small and stays in the caches; the four wavefronts read the same columns).  K in steps of 16, ascending: a
+// row's sums do not depend on what else is in the launch.
+typedef short bf16x4_t __attribute__((ext_vector_type(4)));
+typedef float f32x4_t __attribute__((ext_vector_type(4)));
+
+template <typename TO>
+__global__ __launch_bounds__(256) void linear_heads_kernel(const bf16_t* __restrict__ x, int ldx,
+                                                           const bf16_t* __restrict__ w, TO* __restrict__ out, int ldo,
+                                                           int rows, int N, int K, int ohs) {
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, c = lane & 15, g = lane >> 4;
+  const int h = blockIdx.z, r0 = blockIdx.x * 64 + 16 * wave, n0 = blockIdx.y * 64;
+  if (r0 >= rows) return;
+  const bf16_t* xa = x + (long long)min(r0 + c, rows - 1) * ldx + (long long)h * K + 4 * g;
+  const bf16_t* wb[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) wb[j] = w + ((long long)h * N + min(n0 + 16 * j + c, N - 1)) * K + 4 * g;
+  f32x4_t acc[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) acc[j] = (f32x4_t){0.f, 0.f, 0.f, 0.f};
+  for (int ks = 0; ks < K; ks += 16) {
+    const bf16x4_t a = __builtin_bit_cast(bf16x4_t, *(const uint2*)(xa + ks));
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const bf16x4_t bv = __builtin_bit_cast(bf16x4_t, *(const uint2*)(wb[j] + ks));
+      acc[j] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a, bv, acc[j], 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int n = n0 + 16 * j + c;
+    if (n >= N) continue;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const int r = r0 + 4 * g + e;
+      if (r < rows) out[(long long)r * ldo + (long long)h * ohs + n] = from_f32<TO>(acc[j][e]);
+    }
+  }
+}
+
 }  // namespace
 
 extern "C" int lq_rmsnorm_cols(const float* src, int lds_, const float* w, float eps, void* out, int out_dtype, int ldo,
@@ -92,5 +134,32 @@ extern "C" int lq_rotary(const float* src, int lds_, void* out, int out_dtype, i
                                                             interleaved, freqs, magnitude, row_pos);
   else LQ_REQUIRE(false, "rotary: unknown dtype %d", out_dtype);
   LQ_CHECK_LAUNCH("rotary");
+  return 0;
+}
+
+// Whether lq_linear_heads takes these operands (else the caller runs a product a head).
+extern "C" int lq_linear_heads_accepts(const void* x, const void* w, int in_dtype, int K, int ldx) {
+  return in_dtype == LQ_BF16 && K % 16 == 0 && ldx % 4 == 0 && ((uintptr_t)x % 8) == 0 && ((uintptr_t)w % 8) == 0;
+}
+
+// x [rows, heads * K] (stride ldx), w [heads, N, K] dense, out: head h's N columns from column h * out_head_stride
+extern "C" int lq_linear_heads(const void* x, int ldx, const void* w, void* out, int in_dtype, int out_dtype, int ldo,
+                               int rows, int heads, int N, int K, int out_head_stride, hipStream_t stream) {
+  LQ_REQUIRE(rows > 0 && heads > 0 && heads <= 65535 && N > 0 && K > 0, "linear_heads: rows %d, heads %d, N %d, K %d", rows,
+             heads, N, K);
+  LQ_REQUIRE(ldx >= heads * K && out_head_stride >= N && ldo >= (heads - 1) * out_head_stride + N,
+             "linear_heads: a stride is smaller than what it steps over");
+  LQ_REQUIRE(x && w && out, "linear_heads: null pointer");
+  LQ_REQUIRE(lq_linear_heads_accepts(x, w, in_dtype, K, ldx), "linear_heads: bfloat16 operands, K in 16s, rows on 8 bytes");
+  LQ_REQUIRE(lq_ceil_div(N, 64) <= 65535, "linear_heads: too many columns");
+  dim3 grid(lq_ceil_div(rows, 64), lq_ceil_div(N, 64), heads);
+  if (out_dtype == LQ_F32)
+    linear_heads_kernel<float><<<grid, 256, 0, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, (float*)out, ldo, rows, N, K,
+                                                         out_head_stride);
+  else if (out_dtype == LQ_BF16)
+    linear_heads_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)x, ldx, (const bf16_t*)w, (bf16_t*)out, ldo, rows, N,
+                                                          K, out_head_stride);
+  else LQ_REQUIRE(false, "linear_heads: unknown dtype %d", out_dtype);
+  LQ_CHECK_LAUNCH("linear_heads");
   return 0;
 }

@@ -55,6 +55,76 @@ __global__ __launch_bounds__(256) void moe_glu_kernel(const float* __restrict__ 
   out[r * ldo + i] = from_f32<T>(y);
 }
 
+// ---- a step's rows sorted by expert ----------------------------------------------------------------------------------
+// counts[e] = rows that chose expert e; one workgroup an expert.
+__global__ __launch_bounds__(256) void moe_count_kernel(const float* __restrict__ route, int rows, int E,
+                                                        int* __restrict__ counts) {
+  __shared__ float red[16];
+  const int e = blockIdx.x;
+  float n = 0.f;  // (counts of up to 2^24 rows are whole numbers in 32-bit floats)
+  for (int r = threadIdx.x; r < rows; r += 256) n += route[(long long)r * E + e] >= 0.f ? 1.f : 0.f;
+  n = block_sum(n, red);
+  if (threadIdx.x == 0) counts[e] = (int)n;
+}
+
+// Expert e's rows, in ascending order, take the places offset(e) .. offset(e) + counts[e] - 1 of the sorted list
+// (offset: the counts of the experts before it): order[place] = row, weight[place] = the row's weight for the expert,
+// place_of[row, e] = place (-1 for an expert the row did not choose).  One workgroup an expert walks the rows in
+// chunks of 256 with a running count, so the order does not depend on timing.
+__global__ __launch_bounds__(256) void moe_place_kernel(const float* __restrict__ route, int rows, int E,
+                                                        const int* __restrict__ counts, int* __restrict__ order,
+                                                        float* __restrict__ weight, int* __restrict__ place_of) {
+  __shared__ int wave_n[4];
+  __shared__ int base;
+  const int e = blockIdx.x, lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  if (threadIdx.x == 0) {
+    int off = 0;
+    for (int i = 0; i < e; ++i) off += counts[i];
+    base = off;
+  }
+  __syncthreads();
+  for (int r0 = 0; r0 < rows; r0 += 256) {
+    const int r = r0 + threadIdx.x;
+    const float w = r < rows ? route[(long long)r * E + e] : -1.f;
+    const bool chosen = w >= 0.f;
+    const unsigned long long mask = __ballot(chosen);
+    const int before = __popcll(mask & ((1ull << lane) - 1ull));
+    if (lane == 0) wave_n[wave] = __popcll(mask);
+    __syncthreads();
+    int at = base + before;
+    for (int i = 0; i < wave; ++i) at += wave_n[i];
+    if (chosen) order[at] = r, weight[at] = w;
+    if (r < rows) place_of[(long long)r * E + e] = chosen ? at : -1;
+    __syncthreads();
+    if (threadIdx.x == 0) base += wave_n[0] + wave_n[1] + wave_n[2] + wave_n[3];
+    __syncthreads();
+  }
+}
+
+// dst[i, :] = src[order[i], :] (16-bit or 32-bit rows)
+template <typename T>
+__global__ __launch_bounds__(256) void moe_gather_kernel(const T* __restrict__ src, int lds_, const int* __restrict__ order,
+                                                         T* __restrict__ dst, int width) {
+  const T* s = src + (long long)order[blockIdx.x] * lds_;
+  T* d = dst + (long long)blockIdx.x * width;
+  for (int i = threadIdx.x; i < width; i += 256) d[i] = s[i];
+}
+
+// out[r, :] = the sum, over the experts that row r chose in ascending order, of ys[place_of[r, e], :]
+__global__ __launch_bounds__(256) void moe_scatter_kernel(const float* __restrict__ ys, const int* __restrict__ place_of, int E,
+                                                          float* __restrict__ out, int ldo, int width) {
+  const int r = blockIdx.x;
+  const int* places = place_of + (long long)r * E;
+  for (int i = threadIdx.x; i < width; i += 256) {
+    float acc = 0.f;
+    for (int e = 0; e < E; ++e) {
+      const int at = places[e];
+      if (at >= 0) acc += ys[(long long)at * width + i];
+    }
+    out[(long long)r * ldo + i] = acc;
+  }
+}
+
 }  // namespace
 
 extern "C" int lq_moe_route(const float* z, int ldz, float* route, int rows, int experts, int top, int renormalize,
@@ -85,5 +155,38 @@ extern "C" int lq_moe_glu(const float* gu, long long ldg, const float* route, vo
     else LQ_REQUIRE(false, "moe_glu: unknown dtype %d", out_dtype);
   }
   LQ_CHECK_LAUNCH("moe_glu");
+  return 0;
+}
+
+// route [rows, experts] (a weight, or -1): counts [experts], order and weight [pairs] (pairs: the chosen
+// (row, expert) couples, expert by expert, rows ascending), place_of [rows, experts]
+extern "C" int lq_moe_sort(const float* route, int rows, int experts, int* counts, int* order, float* weight, int* place_of,
+                           hipStream_t stream) {
+  LQ_REQUIRE(rows > 0 && rows < (1 << 24) && experts > 0 && experts <= 65535, "moe_sort: rows %d, experts %d", rows, experts);
+  LQ_REQUIRE(route && counts && order && weight && place_of, "moe_sort: null pointer");
+  moe_count_kernel<<<experts, 256, 0, stream>>>(route, rows, experts, counts);
+  LQ_CHECK_LAUNCH("moe_sort(count)");
+  moe_place_kernel<<<experts, 256, 0, stream>>>(route, rows, experts, counts, order, weight, place_of);
+  LQ_CHECK_LAUNCH("moe_sort(place)");
+  return 0;
+}
+
+extern "C" int lq_moe_gather(const void* src, int dtype, int ld, const int* order, void* dst, int n, int width,
+                             hipStream_t stream) {
+  LQ_REQUIRE(n > 0 && width > 0 && ld >= width, "moe_gather: %d rows of %d (stride %d)", n, width, ld);
+  LQ_REQUIRE(src && order && dst, "moe_gather: null pointer");
+  if (dtype == LQ_F32) moe_gather_kernel<float><<<n, 256, 0, stream>>>((const float*)src, ld, order, (float*)dst, width);
+  else if (dtype == LQ_BF16) moe_gather_kernel<bf16_t><<<n, 256, 0, stream>>>((const bf16_t*)src, ld, order, (bf16_t*)dst, width);
+  else LQ_REQUIRE(false, "moe_gather: unknown dtype %d", dtype);
+  LQ_CHECK_LAUNCH("moe_gather");
+  return 0;
+}
+
+extern "C" int lq_moe_scatter(const float* ys, const int* place_of, int experts, float* out, int ldo, int rows, int width,
+                              hipStream_t stream) {
+  LQ_REQUIRE(rows > 0 && width > 0 && experts > 0 && ldo >= width, "moe_scatter: rows %d, width %d, experts %d", rows, width, experts);
+  LQ_REQUIRE(ys && place_of && out, "moe_scatter: null pointer");
+  moe_scatter_kernel<<<rows, 256, 0, stream>>>(ys, place_of, experts, out, ldo, width);
+  LQ_CHECK_LAUNCH("moe_scatter");
   return 0;
 }

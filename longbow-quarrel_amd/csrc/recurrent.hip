@@ -531,28 +531,35 @@ __global__ __launch_bounds__(TH) void delta_scan_kernel(const float* __restrict_
 // Gated linear attention: S <- diag(a) S + k v^T;  o = S^T (q q_scale), with a decay for every key channel,
 // a = sigmoid(z + bias)^(inv_tau), taken as exp(inv_tau * log sigmoid(z + bias)) in 32-bit.
 // (ScanShape: groups = heads, N = key size, P = value size; the state [slots, heads, P, N].)
-// A chunk of TT tokens is staged in LDS (q, k and the decays of the head, the workgroup's slice of v), computed token
-// by token, and its results leave together.  A token's sums are a thread's own entries in ascending order, then the
-// exchange over the column's lanes: the same in every launch.
+// A chunk of TT tokens is staged in LDS (q, k and the decays of the head, the workgroup's slice of v), two buffers
+// taking turns: the next chunk's loads are in flight while this chunk is computed token by token, and a chunk's
+// results leave together.  A token's sums are a thread's own entries in ascending order, then the exchange over the
+// column's lanes: the same in every launch.
+constexpr int gla_tokens(int np, int th, int ln) {
+  // tokens a chunk: at most 24 registers a thread for the shared rows, and two buffers within 64 KB of LDS
+  const int by_regs = 24 * th / (3 * np), by_lds = 8192 / (3 * np + 2 * (th / ln));
+  const int t = by_regs < by_lds ? by_regs : by_lds;
+  return t >= 16 ? 16 : t >= 8 ? 8 : t >= 4 ? 4 : t >= 2 ? 2 : 1;
+}
+
 template <int LN, int SLAB, int TH>
 __global__ __launch_bounds__(TH) void gla_scan_kernel(const float* __restrict__ q, int ldq, const float* __restrict__ k,
                                                        int ldk, const float* __restrict__ v, int ldv,
                                                        const float* __restrict__ z, int ldz,
                                                        const float* __restrict__ bias, float* __restrict__ state,
                                                        float* __restrict__ out, int ldo, ScanShape sh, float q_scale,
-                                                       float inv_tau, int TT) {
+                                                       float inv_tau) {
   extern __shared__ float lds[];
+  constexpr int NP = LN * SLAB;  // a shared row in LDS, padded with zeros: entries past N take part as zeros
+  constexpr int TT = gla_tokens(NP, TH, LN);
+  constexpr int PER = (3 * TT * NP + TH - 1) / TH;
+  constexpr int cols = TH / LN;
+  constexpr int XPRE = (TT * cols + TH - 1) / TH;
+  constexpr int BUF = TT * (3 * NP + 2 * cols);  // q, k, decays [TT][NP] each, then v and the results [TT][cols]
   const int heads = sh.heads, P = sh.P, N = sh.N;
   const int b = blockIdx.x / heads, h = blockIdx.x % heads;
-  const int threads = blockDim.x, cols = threads / LN, tid = threadIdx.x;
-  const int l = tid % LN, col = tid / LN, p0 = blockIdx.y * cols, p = p0 + col;
+  const int tid = threadIdx.x, l = tid % LN, col = tid / LN, p0 = blockIdx.y * cols, p = p0 + col;
   const bool live = p < P;
-  constexpr int NP = LN * SLAB;  // a shared row in LDS, padded with zeros: entries past N take part as zeros
-  float* qs = lds;               // [TT][NP]
-  float* ks = qs + TT * NP;      // [TT][NP]
-  float* as = ks + TT * NP;      // [TT][NP]
-  float* vs = as + TT * NP;      // [TT][cols]
-  float* os = vs + TT * cols;    // [TT][cols]
   const long long r0 = sh.cu_rows[b], r1 = sh.cu_rows[b + 1];
   float* sp = state + (((long long)sh.seq_slot[b] * heads + h) * P + (live ? p : 0)) * N;
   float S[SLAB];
@@ -561,36 +568,72 @@ __global__ __launch_bounds__(TH) void gla_scan_kernel(const float* __restrict__ 
     const int n = i * LN + l;
     S[i] = (live && n < N) ? sp[n] : 0.f;
   }
-  for (int e = tid; e < 3 * TT * NP; e += threads) lds[e] = 0.f;
-  __syncthreads();
-  for (long long c0 = r0; c0 < r1; c0 += TT) {
-    const int nt = (int)min((long long)TT, r1 - c0);
-    for (int e = tid; e < nt * N; e += threads) {
-      const int t = e / N, n = e - t * N;
-      const long long r = c0 + t;
-      qs[t * NP + n] = q[r * ldq + h * N + n] * q_scale;
-      ks[t * NP + n] = k[r * ldk + h * N + n];
-      as[t * NP + n] = expf(-softplus_f(-(z[r * ldz + h * N + n] + bias[h * N + n])) * inv_tau);
-    }
-    for (int e = tid; e < nt * cols; e += threads) {
-      const int t = e / cols, c = e - t * cols;
-      vs[e] = p0 + c < P ? v[(c0 + t) * ldv + h * P + p0 + c] : 0.f;
-    }
-    __syncthreads();
-    for (int t = 0; t < nt; ++t) {
-      const float vv = vs[t * cols + col];
-      float acc = 0.f;
+  float pre[PER], xpre[XPRE];
+  auto fetch = [&](long long c0, int nt) {  // the chunk's loads, into registers
 #pragma unroll
-      for (int i = 0; i < SLAB; ++i) {
+    for (int j = 0; j < PER; ++j) {
+      const int e = tid + j * TH, which = e / (TT * NP), rem = e - which * (TT * NP), t = rem / NP, n = rem - t * NP;
+      float val = 0.f;
+      if (which < 3 && t < nt && n < N) {
+        const long long r = c0 + t;
+        val = which == 0 ? q[r * ldq + h * N + n] : which == 1 ? k[r * ldk + h * N + n] : z[r * ldz + h * N + n];
+      }
+      pre[j] = val;
+    }
+#pragma unroll
+    for (int j = 0; j < XPRE; ++j) {
+      const int e = tid + j * TH, t = e / cols, c = e - t * cols;
+      xpre[j] = (t < nt && p0 + c < P) ? v[(c0 + t) * ldv + h * P + p0 + c] : 0.f;
+    }
+  };
+  auto stash = [&](float* buf) {  // registers to LDS; the decay is made of its logit here
+#pragma unroll
+    for (int j = 0; j < PER; ++j) {
+      const int e = tid + j * TH, which = e / (TT * NP), n = e % NP;
+      if (which >= 3) continue;
+      float val = pre[j];
+      if (which == 0) val *= q_scale;
+      else if (which == 2) val = n < N ? expf(-softplus_f(-(val + bias[h * N + n])) * inv_tau) : 0.f;
+      buf[e] = val;
+    }
+#pragma unroll
+    for (int j = 0; j < XPRE; ++j) {
+      const int e = tid + j * TH;
+      if (e < TT * cols) buf[3 * TT * NP + e] = xpre[j];
+    }
+  };
+  int cur = 0;
+  if (r1 > r0) {
+    fetch(r0, (int)min((long long)TT, r1 - r0));
+    stash(lds);
+  }
+  __syncthreads();
+  for (long long c0 = r0; c0 < r1; c0 += TT, cur ^= 1) {
+    const int nt = (int)min((long long)TT, r1 - c0);
+    const int next = (int)min((long long)TT, r1 - c0 - TT);
+    if (next > 0) fetch(c0 + TT, next);
+    float* buf = lds + cur * BUF;
+    const float *qs = buf, *ks = buf + TT * NP, *as = buf + 2 * TT * NP, *vs = buf + 3 * TT * NP;
+    float* os = buf + 3 * TT * NP + TT * cols;
+#pragma unroll
+    for (int t = 0; t < TT; ++t) {
+      if (t >= nt) break;
+      const float vv = vs[t * cols + col];
+      float acc = 0.f, acc1 = 0.f;
+#pragma unroll
+      for (int i = 0; i < SLAB; i += 2) {
         const int n = t * NP + i * LN + l;
         S[i] = fmaf(ks[n], vv, as[n] * S[i]);
+        S[i + 1] = fmaf(ks[n + LN], vv, as[n + LN] * S[i + 1]);
         acc = fmaf(S[i], qs[n], acc);
+        acc1 = fmaf(S[i + 1], qs[n + LN], acc1);
       }
-      acc = group_sum<LN>(acc);
+      acc = group_sum<LN>(acc + acc1);
       if (l == 0) os[t * cols + col] = acc;
     }
+    if (next > 0) stash(lds + (cur ^ 1) * BUF);
     __syncthreads();
-    for (int e = tid; e < nt * cols; e += threads) {
+    for (int e = tid; e < nt * cols; e += TH) {
       const int t = e / cols, c = e - t * cols;
       if (p0 + c < P) out[(c0 + t) * ldo + h * P + p0 + c] = os[e];
     }
@@ -917,15 +960,13 @@ extern "C" int lq_gla_scan(const float* q, int ldq, const float* k, int ldk, con
   ScanLaunch cfg;
   LQ_REQUIRE(scan_launch(Dk, P, (long long)batch * heads, cfg), "gla_scan: key size %d is too large", Dk);
   const int np = cfg.ln * cfg.slab;
-  int tt = 8;
-  while (tt > 1 && (size_t)tt * (3 * np + 2 * cfg.cols) * sizeof(float) > 64 * 1024) tt >>= 1;
-  const size_t lds = (size_t)tt * (3 * np + 2 * cfg.cols) * sizeof(float);
+  const size_t lds = 2 * (size_t)gla_tokens(np, cfg.threads, cfg.ln) * (3 * np + 2 * cfg.cols) * sizeof(float);
   LQ_REQUIRE(lds <= 64 * 1024, "gla_scan: key size %d is too large", Dk);
   dim3 grid((unsigned)(batch * heads), lq_ceil_div(P, cfg.cols));
   ScanShape sh = {heads, heads, P, Dk, seq_slot, cu_rows};
 #define LQ_GLA(LN, SL, TH)                                                                                            \
   gla_scan_kernel<LN, SL, TH><<<grid, cfg.threads, lds, stream>>>(q, ldq, k, ldk, v, ldv, z, ldz, bias, state, out, ldo, \
-                                                                  sh, q_scale, inv_tau, tt)
+                                                                  sh, q_scale, inv_tau)
   LQ_SCAN_LANES(LQ_GLA)
 #undef LQ_GLA
   LQ_CHECK_LAUNCH("gla_scan");

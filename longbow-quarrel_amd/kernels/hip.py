@@ -966,7 +966,8 @@ class HipKernels:
                                        self.stream))
 
     def linear_heads(self, x: torch.Tensor, w: torch.Tensor, out: torch.Tensor, heads: int, out_head_stride: int) -> None:
-        """A product a head: out[r, h out_head_stride .. + N) = x[r, h K .. + K) . w[h]^T with w [heads, N, K]."""
+        """A product a head: out[r, h out_head_stride .. + N) = x[r, h K .. + K) . w[h]^T with w [heads, N, K]: one
+        launch for bfloat16 operands with K in 16s, else a product a head."""
         rows, kx, ldx = self._mat(x, "linear_heads: x")
         ro, no, ldc = self._mat(out, "linear_heads: out")
         if w.dim() != 3 or not w.is_contiguous() or not w.is_cuda or w.shape[0] != heads or kx != heads * w.shape[2] \
@@ -974,6 +975,11 @@ class HipKernels:
                 or x.dtype != w.dtype:
             raise KernelLibraryError(f"linear_heads: x {tuple(x.shape)}, w {tuple(w.shape)}, out {tuple(out.shape)} do not fit")
         n, k = int(w.shape[1]), int(w.shape[2])
+        if not self.force_generic and self.lib.lq_linear_heads_accepts(_ptr(x), _ptr(w), c_int(_code(x)), c_int(k), c_int(ldx)):
+            self._check(self.lib.lq_linear_heads(_ptr(x), c_int(ldx), _ptr(w), _ptr(out), c_int(_code(x)), c_int(_code(out)),
+                                                 c_int(ldc), c_int(rows), c_int(heads), c_int(n), c_int(k),
+                                                 c_int(out_head_stride), self.stream))
+            return
         xe, we, oe = x.element_size(), w.element_size(), out.element_size()
         cx, co = _code(x), _code(out)
         generic = 1 if self.force_generic else 0
@@ -1032,6 +1038,55 @@ class HipKernels:
         self._check(self.lib.lq_moe_glu(_ptr(gu), c_longlong(ldg), _ptr(route), _ptr(out), c_int(_code(out)),
                                         c_longlong(ldo), c_int(rows), c_int(experts), c_int(ff), c_float(limit),
                                         c_int(1 if weight_input else 0), self.stream))
+
+    def weight_rows(self, w, start: int, n: int):
+        """Rows start .. start + n of a product weight as a weight of its own: a view of a dense one; of a packed
+        one the same run of its memory, where the rows are whole groups of eight and a matrix of that size is
+        packed at all (else None: the caller keeps the weight dense)."""
+        if not getattr(w, "packed", False):
+            return w[start : start + n]
+        rows, k = w.shape
+        if start % 8 or n % 8 or start + n > rows or \
+                not self.lib.lq_weight_packable(c_int(_DTYPE_CODE[w.dtype]), c_int(n), c_int(k)):
+            return None
+        return PackedWeight(w.data.view(-1)[start * k : (start + n) * k].view(n, k), n, k)
+
+    def moe_sort(self, route: torch.Tensor, counts: torch.Tensor, order: torch.Tensor, weight: torch.Tensor,
+                 place_of: torch.Tensor) -> None:
+        """The chosen (row, expert) couples of route [rows, experts] (a weight, or -1), expert by expert with rows
+        ascending: counts[e] rows of expert e, order[place] = row, weight[place] = its weight, place_of[row, e] =
+        place or -1."""
+        rows, experts = route.shape
+        self._f32(route, "moe_sort: route", rows * experts)
+        self._f32(weight, "moe_sort: weight")
+        self._i32(counts, "counts", experts)
+        self._i32(place_of, "place_of", rows * experts)
+        if order.dtype != torch.int32 or not order.is_contiguous() or not weight.is_contiguous() \
+                or order.numel() != weight.numel() or order.numel() < rows:
+            raise KernelLibraryError("moe_sort: order (int32) and weight (float32) hold a place for every chosen couple")
+        self._dev(route, counts, order, weight, place_of)
+        self._check(self.lib.lq_moe_sort(_ptr(route), c_int(rows), c_int(experts), _ptr(counts), _ptr(order), _ptr(weight),
+                                         _ptr(place_of), self.stream))
+
+    def moe_gather(self, src: torch.Tensor, order: torch.Tensor, dst: torch.Tensor, n: int) -> None:
+        """dst[i] = src[order[i]] for the first n places."""
+        rows, width, ld = self._mat(src, "moe_gather: src")
+        if dst.dtype != src.dtype or dst.dim() != 2 or dst.shape[1] != width or not dst.is_contiguous() or dst.shape[0] < n \
+                or order.numel() < n or order.dtype != torch.int32 or not dst.is_cuda:
+            raise KernelLibraryError("moe_gather: dst dense [>= n, width] in the dtype of src, order int32")
+        self._check(self.lib.lq_moe_gather(_ptr(src), c_int(_code(src)), c_int(ld), _ptr(order), _ptr(dst), c_int(n),
+                                           c_int(width), self.stream))
+
+    def moe_scatter(self, ys: torch.Tensor, place_of: torch.Tensor, out: torch.Tensor) -> None:
+        """out[r] = the sum over the experts e that row r chose, in ascending order, of ys[place_of[r, e]]."""
+        rows, width, ldo = self._mat(out, "moe_scatter: out")
+        self._f32(ys, "moe_scatter: ys")
+        self._f32(out, "moe_scatter: out")
+        if place_of.dtype != torch.int32 or place_of.dim() != 2 or place_of.shape[0] != rows or not place_of.is_contiguous() \
+                or ys.dim() != 2 or ys.shape[1] != width or not ys.is_contiguous():
+            raise KernelLibraryError("moe_scatter: ys dense [places, width], place_of int32 [rows, experts]")
+        self._check(self.lib.lq_moe_scatter(_ptr(ys), _ptr(place_of), c_int(place_of.shape[1]), _ptr(out), c_int(ldo),
+                                            c_int(rows), c_int(width), self.stream))
 
     # ------------------------------------------------------------------ sampling
     @property

@@ -122,7 +122,7 @@ class GatedLinearUnit(FeedForward):
 class MixtureOfExperts(FeedForward):
     """`experts` small gated feed-forwards of which every token uses `top`, chosen by a router.
 
-    Router: z = Wr h in 32-bit, s = sigmoid(z); the `top` largest scores win (the lower index on a tie); an expert's
+    Router: z = Wr h summed in 32-bit (h as the run holds it), s = sigmoid(z) in 32-bit; the `top` largest scores win (the lower index on a tie); an expert's
     weight is its score as it is (`renormalize` divides the chosen scores by their sum).  With `weight_input` the
     weight multiplies what the expert reads, out = sum_e expert_e(s_e h); otherwise its result.
 
@@ -132,12 +132,17 @@ class MixtureOfExperts(FeedForward):
 
     How it runs.  The experts' gate and up matrices are one matrix [experts * 2 ff, width] and their down matrices
     one [width, experts * ff]: with the activations of the experts that a token did not choose set to zero, the down
-    product adds the chosen experts' results by itself.  Every row runs through all experts' columns: a decoding
-    batch of more than a few tokens reads nearly all experts anyway; a prompt pays experts / top times the
-    arithmetic of a step whose rows are sorted by expert, which is not built."""
+    product adds the chosen experts' results by itself.  A step of few rows (decoding) runs every row through all
+    experts' columns: a batch of more than a few tokens reads nearly all experts anyway.  A prompt step of
+    `sort_from_rows` rows or more is sorted by expert first (`moe_sort`: the chosen (row, expert) couples expert by
+    expert, rows ascending), the rows gathered in that order, and every expert's two products run over its own rows
+    only; the results go back to their rows and are added in the order of the experts.  The host reads the experts'
+    row counts for that (one wait a layer), which a captured step never does: it takes the first way."""
 
     graph_safe = True
     takes_out = True
+    #: rows from which a step that is no decoding step is sorted by expert
+    sort_from_rows = 256
 
     def __init__(self, width: int, experts: int, top: int, inner: int, limit: float, prefix: str,
                  weight_input: bool = True, renormalize: bool = False, names: Optional[Mapping[str, str]] = None) -> None:
@@ -168,9 +173,23 @@ class MixtureOfExperts(FeedForward):
         if len({m.dtype for m in gu + down}) != 1:
             raise ValueError(f"{self._name(0, 'gate')}: the experts' matrices are stored in different dtypes")
         # expert e's rows of the first matrix: [gate (ff) | up (ff)]; its columns of the second: e ff .. (e + 1) ff
-        self.w_gate_up = product_weight(env, torch.cat(gu, dim=0))  # [E * 2 ff, width]
-        self.w_down = product_weight(env, torch.cat(down, dim=1))   # [width, E * ff]
-        self.w_router = tensors[f"{self.prefix}.{self.n['router']}"].float().contiguous()  # the router is 32-bit
+        ff = self.inner
+        whole = torch.cat(gu, dim=0).contiguous()  # [E * 2 ff, width]
+        self.w_gate_up = product_weight(env, whole)
+        rows_of = getattr(env.kernels, "weight_rows", None)
+        if self.w_gate_up is whole:
+            self.gate_up_of = [whole[e * 2 * ff : (e + 1) * 2 * ff] for e in range(E)]
+        else:  # held in the products' own order: an expert's rows must be a weight in that order too
+            self.gate_up_of = [rows_of(self.w_gate_up, e * 2 * ff, 2 * ff) if rows_of else None for e in range(E)]
+            if any(w is None for w in self.gate_up_of):
+                self.w_gate_up = whole
+                self.gate_up_of = [whole[e * 2 * ff : (e + 1) * 2 * ff] for e in range(E)]
+        # the second matrix stays dense: an expert is a run of its columns, which only the dense order can give
+        self.w_down = torch.cat(down, dim=1).contiguous()  # [width, E * ff]
+        self.down_of = [self.w_down[:, e * ff : (e + 1) * ff] for e in range(E)]
+        # the router's product as it is stored: bfloat16 operands multiply exactly into 32-bit sums, and its result
+        # (the logits) and everything after it are 32-bit
+        self.w_router = tensors[f"{self.prefix}.{self.n['router']}"].contiguous()
 
     def forward(self, h, ctx: StepContext, out: Optional[torch.Tensor] = None) -> torch.Tensor:
         kn = ctx.kernels
@@ -181,9 +200,46 @@ class MixtureOfExperts(FeedForward):
         kn.moe_route(z, route, self.top, self.renormalize)
         if out is None:
             out = ctx.ws.alloc((rows, self.width), torch.float32)
+        if rows >= self.sort_from_rows and not ctx.decode and not ctx.dry and E > self.top \
+                and getattr(kn, "moe_sort", None) is not None:
+            self._sorted(h, route, out, ctx)
+            return out
         gu = ctx.ws.alloc((rows, E * 2 * ff), torch.float32)
         project(kn, ctx, h, self.w_gate_up, gu)
         act = ctx.ws.alloc((rows, E * ff), ctx.dtype)
         kn.moe_glu(gu, route, act, E, ff, self.limit, self.weight_input)
         project(kn, ctx, act, self.w_down, out)
         return out
+
+    def _sorted(self, h, route, out, ctx: StepContext) -> None:
+        """The step's rows sorted by expert: every expert's products over its own rows only."""
+        kn = ctx.kernels
+        rows, E, ff, top = h.shape[0], self.experts, self.inner, self.top
+        pairs = rows * top
+        counts = ctx.ws.alloc((E,), torch.int32)
+        order = ctx.ws.alloc((pairs,), torch.int32)       # sorted place -> row
+        weight = ctx.ws.alloc((pairs, 1), torch.float32)  # sorted place -> the row's weight for its expert
+        place_of = ctx.ws.alloc((rows, E), torch.int32)   # (row, expert) -> sorted place, or -1
+        kn.moe_sort(route, counts, order, weight, place_of)
+        n_of = counts.tolist()  # the one wait: the products below are launched with every expert's number of rows
+        total = sum(n_of)
+        if total == 0:
+            kn.moe_scatter(out, place_of, out)  # (no row chose anything: zeros)
+            return
+        hs = ctx.ws.alloc((pairs, self.width), h.dtype)
+        kn.moe_gather(h, order, hs, total)
+        gu = ctx.ws.alloc((pairs, 2 * ff), torch.float32)
+        at = 0
+        for e, n in enumerate(n_of):
+            if n:
+                project(kn, ctx, hs[at : at + n], self.gate_up_of[e], gu[at : at + n])
+                at += n
+        act = ctx.ws.alloc((pairs, ff), ctx.dtype)
+        kn.moe_glu(gu[:total], weight[:total], act[:total], 1, ff, self.limit, self.weight_input)
+        ys = ctx.ws.alloc((pairs, self.width), torch.float32)
+        at = 0
+        for e, n in enumerate(n_of):
+            if n:
+                project(kn, ctx, act[at : at + n], self.down_of[e], ys[at : at + n])
+                at += n
+        kn.moe_scatter(ys, place_of, out)

@@ -340,3 +340,23 @@ class CpuKernels:
             y = y * w
         y = torch.where(w >= 0, y, torch.zeros_like(y))
         out.copy_(y.reshape(rows, experts * ff).to(out.dtype))
+
+    def moe_sort(self, route, counts, order, weight, place_of):
+        rows, experts = route.shape
+        place_of.fill_(-1)
+        at = 0
+        for e in range(experts):
+            mine = [r for r in range(rows) if float(route[r, e]) >= 0]
+            counts[e] = len(mine)
+            for r in mine:
+                order[at], weight.view(-1)[at], place_of[r, e] = r, route[r, e], at
+                at += 1
+
+    def moe_gather(self, src, order, dst, n):
+        dst[:n] = src[order[:n].long()]
+
+    def moe_scatter(self, ys, place_of, out):
+        out.zero_()
+        for e in range(place_of.shape[1]):
+            at = place_of[:, e].long()
+            out += torch.where((at >= 0)[:, None], ys[at.clamp(min=0)], torch.zeros_like(out))

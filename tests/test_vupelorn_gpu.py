@@ -127,8 +127,9 @@ def test_norm_over_columns_rotation_and_the_norm_of_a_result(kn, dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-def test_products_a_head(kn, dtype):
-    rows, heads, k, n, stride = 21, 5, 24, 13, 19
+@pytest.mark.parametrize("sizes", [(21, 5, 24, 13, 19), (21, 5, 32, 13, 19), (150, 3, 128, 192, 256), (1, 2, 16, 70, 70)])
+def test_products_a_head(kn, dtype, sizes):
+    rows, heads, k, n, stride = sizes
     x, w = rnd(rows, heads * k, seed=1).to(dtype), rnd(heads, n, k, seed=2).to(dtype)
     out = torch.zeros(rows, heads * stride + 3, dtype=dtype, device=DEV)
     kn.linear_heads(dev(x, dtype), dev(w, dtype), out[:, 3:], heads, stride)
