@@ -615,21 +615,42 @@ __global__ __launch_bounds__(TH) void gla_scan_kernel(const float* __restrict__ 
     float* buf = lds + cur * BUF;
     const float *qs = buf, *ks = buf + TT * NP, *as = buf + 2 * TT * NP, *vs = buf + 3 * TT * NP;
     float* os = buf + 3 * TT * NP + TT * cols;
+    // a token's operands are read from LDS into registers while the token before it is computed (two sets of
+    // registers take turns: a read placed after the LDS store of a result could not pass it)
+    struct Tok {
+      float q[SLAB], k[SLAB], a[SLAB], v;
+    };
+    auto load = [&](Tok& x, int t) {
+      x.v = vs[t * cols + col];
 #pragma unroll
-    for (int t = 0; t < TT; ++t) {
-      if (t >= nt) break;
-      const float vv = vs[t * cols + col];
-      float acc = 0.f, acc1 = 0.f;
+      for (int i = 0; i < SLAB; ++i) {
+        const int n = t * NP + i * LN + l;
+        x.q[i] = qs[n], x.k[i] = ks[n], x.a[i] = as[n];
+      }
+    };
+    auto compute = [&](const Tok& x, int t) {
+      float acc = 0.f, acc1 = 0.f;  // (two chains of multiply-adds, even and odd entries, added at the end)
 #pragma unroll
       for (int i = 0; i < SLAB; i += 2) {
-        const int n = t * NP + i * LN + l;
-        S[i] = fmaf(ks[n], vv, as[n] * S[i]);
-        S[i + 1] = fmaf(ks[n + LN], vv, as[n + LN] * S[i + 1]);
-        acc = fmaf(S[i], qs[n], acc);
-        acc1 = fmaf(S[i + 1], qs[n + LN], acc1);
+        S[i] = fmaf(x.k[i], x.v, x.a[i] * S[i]);
+        S[i + 1] = fmaf(x.k[i + 1], x.v, x.a[i + 1] * S[i + 1]);
+        acc = fmaf(S[i], x.q[i], acc);
+        acc1 = fmaf(S[i + 1], x.q[i + 1], acc1);
       }
       acc = group_sum<LN>(acc + acc1);
       if (l == 0) os[t * cols + col] = acc;
+    };
+    Tok ta, tb;
+    load(ta, 0);
+#pragma unroll
+    for (int t = 0; t < TT; t += 2) {  // (unrolled: a token's places in LDS are constants)
+      if (t >= nt) break;
+      if (t + 1 < nt) load(tb, t + 1);
+      compute(ta, t);
+      if (t + 1 < nt) {
+        if (t + 2 < nt) load(ta, t + 2);
+        compute(tb, t + 1);
+      }
     }
     if (next > 0) stash(lds + (cur ^ 1) * BUF);
     __syncthreads();

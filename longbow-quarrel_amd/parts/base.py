@@ -568,3 +568,4 @@ def project(kn, ctx: StepContext, x: torch.Tensor, w: torch.Tensor, out: torch.T
     wide = ctx.ws.alloc(x.shape, torch.float32)
     kn.cast(x, wide)
     kn.linear(wide, w, out)
+

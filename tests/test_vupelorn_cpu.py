@@ -210,6 +210,16 @@ def test_slots_and_blocks_are_freed_and_used_again(cases, name):
     uc.slots_and_blocks_used_again(cases(name), TOL)
 
 
+@pytest.mark.parametrize("name", ["a", "moe"])
+def test_prompt_rows_sorted_by_expert(cases, name, monkeypatch):
+    """A prompt step of many rows sorts them by expert and runs every expert over its own rows: the same logits."""
+    from longbow_quarrel_amd.parts.feedforward import MixtureOfExperts
+    monkeypatch.setattr(MixtureOfExperts, "sort_from_rows", 2)
+    case = cases(name)
+    t = uc.tokens(90, case.vocab, 12)
+    assert uc.err(case.run_cut(t, [50, 3, 30]), case.want(t)) < TOL
+
+
 def test_the_residual_stream_after_every_layer(cases):
     case = cases("a")
     got, want = case.layers(uc.tokens(37, case.vocab, 8))

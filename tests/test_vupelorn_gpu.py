@@ -167,6 +167,41 @@ def test_router_and_experts_activation(kn):
         assert uc.err(out.cpu(), want) < TOL_F32
 
 
+def test_rows_sorted_by_expert_and_back(kn):
+    rows, E, width = 300, 5, 40
+    route = torch.where(rnd(rows, E, seed=1) > 0.3, rnd(rows, E, seed=2).abs(), torch.full((rows, E), -1.0))
+    route[7] = -1.0  # a row that chose nothing
+    pairs = int((route >= 0).sum())
+    counts, order = torch.zeros(E, dtype=torch.int32, device=DEV), torch.full((rows * E,), -7, dtype=torch.int32, device=DEV)
+    weight, place_of = torch.zeros(rows * E, 1, device=DEV), torch.zeros(rows, E, dtype=torch.int32, device=DEV)
+    kn.moe_sort(dev(route), counts, order, weight, place_of)
+    assert counts.tolist() == (route >= 0).sum(0).tolist()
+    want_order = [r for e in range(E) for r in range(rows) if route[r, e] >= 0]
+    assert order[:pairs].tolist() == want_order and bool((order[pairs:] == -7).all())
+    want_w = [float(route[r, e]) for e in range(E) for r in range(rows) if route[r, e] >= 0]
+    assert weight[:pairs, 0].tolist() == want_w
+    at = 0
+    for e in range(E):
+        for r in range(rows):
+            if route[r, e] >= 0:
+                assert int(place_of[r, e]) == at
+                at += 1
+            else:
+                assert int(place_of[r, e]) == -1
+    for dtype in (torch.float32, torch.bfloat16):
+        src = rnd(rows, width + 8, seed=3).to(dtype)
+        dst = torch.zeros(rows * E, width, dtype=dtype, device=DEV)
+        kn.moe_gather(dev(src, dtype)[:, :width], order, dst, pairs)
+        assert torch.equal(dst[:pairs].cpu(), src[want_order, :width]) and bool((dst[pairs:] == 0).all())
+    ys = rnd(pairs, width, seed=4)
+    out = torch.full((rows, width), 9.0, device=DEV)
+    kn.moe_scatter(dev(ys), place_of, out)
+    want = torch.zeros(rows, width, dtype=torch.float64)
+    for i, r in enumerate(want_order):
+        want[r] += ys[i].double()
+    assert uc.err(out.cpu(), want) < 1e-6 and bool((out[7] == 0).all())
+
+
 def test_bigram_rows_and_the_token_kept_between_steps(kn):
     width, buckets, vocab = 24, 11, 50
     table = rnd(buckets + 1, width, seed=1)
@@ -215,6 +250,22 @@ def test_float32_under_every_cutting_and_batching(cases, name):
     uc.portions(case, TOL_F32)
     uc.unequal_batches(case, TOL_F32)
     uc.slots_and_blocks_used_again(case, TOL_F32)
+
+
+@pytest.mark.parametrize("name,dtype", [("a", "float32"), ("c", "float32"), ("c", "bfloat16")])
+def test_prompt_rows_sorted_by_expert(cases, name, dtype, monkeypatch):
+    """The same logits whether a prompt's rows run through all experts' columns or are sorted by expert."""
+    from longbow_quarrel_amd.parts.feedforward import MixtureOfExperts
+    case = cases(name, dtype)
+    t = uc.tokens(300, case.vocab, 12)
+    monkeypatch.setattr(MixtureOfExperts, "sort_from_rows", 10 ** 9)
+    every = case.run_cut(t, [300])
+    monkeypatch.setattr(MixtureOfExperts, "sort_from_rows", 2)
+    by_expert = case.run_cut(t, [200, 3, 90])
+    if dtype == "float32":
+        assert uc.err(by_expert, case.want(t)) < TOL_F32 and uc.err(by_expert, every) < TOL_F32
+    else:
+        uc.assert_close_bf16(by_expert, case.want(t), case.noise(t))
 
 
 def test_the_residual_stream_after_every_layer(cases):
