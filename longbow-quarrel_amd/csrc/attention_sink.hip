@@ -236,7 +236,7 @@ __global__ __launch_bounds__(64 * SPLIT) void sink_tiles_kernel(const T* __restr
 
 // Any sizes: one wavefront per (row, head), a lane a key of the chunk for the scores and a value dimension (or
 // several) for the sums.
-constexpr int MAX_DIM = 512;
+constexpr int MAX_DIM = 1024;
 
 template <typename T>
 __global__ __launch_bounds__(64) void sink_rows_kernel(const T* __restrict__ q, T* __restrict__ out,

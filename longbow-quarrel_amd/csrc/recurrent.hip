@@ -548,7 +548,7 @@ __global__ __launch_bounds__(TH) void gla_scan_kernel(const float* __restrict__ 
                                                        const float* __restrict__ z, int ldz,
                                                        const float* __restrict__ bias, float* __restrict__ state,
                                                        float* __restrict__ out, int ldo, ScanShape sh, float q_scale,
-                                                       float inv_tau) {
+                                                       float inv_tau, SegArgs sg) {
   extern __shared__ float lds[];
   constexpr int NP = LN * SLAB;  // a shared row in LDS, padded with zeros: entries past N take part as zeros
   constexpr int TT = gla_tokens(NP, TH, LN);
@@ -560,13 +560,29 @@ __global__ __launch_bounds__(TH) void gla_scan_kernel(const float* __restrict__ 
   const int b = blockIdx.x / heads, h = blockIdx.x % heads;
   const int tid = threadIdx.x, l = tid % LN, col = tid / LN, p0 = blockIdx.y * cols, p = p0 + col;
   const bool live = p < P;
-  const long long r0 = sh.cu_rows[b], r1 = sh.cu_rows[b + 1];
+  long long r0 = sh.cu_rows[b], r1 = sh.cu_rows[b + 1];
+  // A long sequence of a launch in segments (see SegArgs; here a segment leaves the product of its decays for
+  // every key channel): this workgroup's segment, where it starts from and where it leaves its state.
+  const int seg = blockIdx.z;
+  const int nseg = (sg.nseg > 1 && r1 - r0 >= SEG_MIN_ROWS) ? sg.nseg : 1;
+  if (seg >= nseg || (sg.pass == 2 && seg == 0)) return;
+  if (nseg > 1) {
+    const long long len = ((r1 - r0 + nseg - 1) / nseg + TT - 1) / TT * TT;
+    r0 = min(r1, r0 + seg * len);
+    r1 = min(r1, r0 + len);
+  }
+  const bool write_out = sg.pass == 2 || seg == 0;
   float* sp = state + (((long long)sh.seq_slot[b] * heads + h) * P + (live ? p : 0)) * N;
-  float S[SLAB];
+  float* seg_sp = nseg > 1 ? sg.state + ((((long long)blockIdx.x * sg.nseg + seg) * P + (live ? p : 0)) * N) : nullptr;
+  const float* from = nseg > 1 && sg.pass == 2 ? seg_sp : sp;
+  const bool from_zero = nseg > 1 && sg.pass == 1 && seg > 0;
+  float* to = nseg == 1 ? sp : sg.pass == 1 ? seg_sp : nullptr;
+  float S[SLAB], aprod[SLAB];  // aprod: the product of the segment's decays of this thread's channels
 #pragma unroll
   for (int i = 0; i < SLAB; ++i) {
     const int n = i * LN + l;
-    S[i] = (live && n < N) ? sp[n] : 0.f;
+    S[i] = (live && !from_zero && n < N) ? from[n] : 0.f;
+    aprod[i] = 1.f;
   }
   float pre[PER], xpre[XPRE];
   auto fetch = [&](long long c0, int nt) {  // the chunk's loads, into registers
@@ -637,6 +653,10 @@ __global__ __launch_bounds__(TH) void gla_scan_kernel(const float* __restrict__ 
         acc = fmaf(S[i], x.q[i], acc);
         acc1 = fmaf(S[i + 1], x.q[i + 1], acc1);
       }
+      if (from_zero) {
+#pragma unroll
+        for (int i = 0; i < SLAB; ++i) aprod[i] *= x.a[i];
+      }
       acc = group_sum<LN>(acc + acc1);
       if (l == 0) os[t * cols + col] = acc;
     };
@@ -654,18 +674,47 @@ __global__ __launch_bounds__(TH) void gla_scan_kernel(const float* __restrict__ 
     }
     if (next > 0) stash(lds + (cur ^ 1) * BUF);
     __syncthreads();
-    for (int e = tid; e < nt * cols; e += TH) {
-      const int t = e / cols, c = e - t * cols;
-      if (p0 + c < P) out[(c0 + t) * ldo + h * P + p0 + c] = os[e];
-    }
+    if (write_out)
+      for (int e = tid; e < nt * cols; e += TH) {
+        const int t = e / cols, c = e - t * cols;
+        if (p0 + c < P) out[(c0 + t) * ldo + h * P + p0 + c] = os[e];
+      }
   }
-  if (live) {
+  if (live && to != nullptr) {
 #pragma unroll
     for (int i = 0; i < SLAB; ++i) {
       const int n = i * LN + l;
-      if (n < N) sp[n] = S[i];
+      if (n < N) to[n] = S[i];
     }
   }
+  if (from_zero && col == 0 && blockIdx.y == 0) {
+#pragma unroll
+    for (int i = 0; i < SLAB; ++i) {
+      const int n = i * LN + l;
+      if (n < N) sg.decay[((long long)blockIdx.x * sg.nseg + seg) * N + n] = aprod[i];
+    }
+  }
+}
+
+// Between the two passes of a gated-linear-attention launch in segments: segment 0 left the state at its true end,
+// every other segment the state it reaches from zero and, for every key channel, the product of its decays.  In
+// order, every segment's true start takes the place of what it left, and the last segment's true end goes into the
+// cache.
+__global__ __launch_bounds__(256) void gla_chain_kernel(float* __restrict__ state, int heads, int P, int N, SegArgs sg,
+                                                        const int* __restrict__ seq_slot, const int* __restrict__ cu_rows) {
+  const int b = blockIdx.x / heads, h = blockIdx.x % heads;
+  if (cu_rows[b + 1] - cu_rows[b] < SEG_MIN_ROWS) return;
+  const long long PN = (long long)P * N, idx = (long long)blockIdx.y * 256 + threadIdx.x;
+  if (idx >= PN) return;
+  const int n = (int)(idx % N);
+  float* segs = sg.state + (long long)blockIdx.x * sg.nseg * PN + idx;
+  float cur = segs[0];
+  for (int s = 1; s < sg.nseg; ++s) {
+    const float reached = segs[s * PN], a = sg.decay[((long long)blockIdx.x * sg.nseg + s) * N + n];
+    segs[s * PN] = cur;
+    cur = fmaf(a, cur, reached);
+  }
+  state[((long long)seq_slot[b] * heads + h) * PN + idx] = cur;
 }
 
 // ---------------------------------------------------------------- norms after the scans
@@ -969,27 +1018,59 @@ extern "C" int lq_rmsnorm_mean(const float* stack, int n_in, const float* w0, co
   return 0;
 }
 
+// Whether a gated-linear-attention launch runs in segments, and then the float32 scratch it needs (as for the
+// state-space scan: few long sequences that would leave most of the chip idle).
+static long long gla_segment_floats(int batch, int heads, int P, int N, int max_rows) {
+  ScanLaunch cfg;
+  if (max_rows < SEG_MIN_ROWS || !scan_launch(N, P, 1ll << 40, cfg)) return 0;
+  if ((long long)batch * heads * lq_ceil_div(P, cfg.cols) >= 4ll * lq_compute_units()) return 0;
+  return (long long)batch * heads * SEG_COUNT * ((long long)P * N + N);
+}
+
+extern "C" long long lq_gla_scan_workspace(int batch, int heads, int P, int N, int max_rows) {
+  if (batch <= 0 || heads <= 0 || P <= 0 || N <= 0) return 0;
+  return gla_segment_floats(batch, heads, P, N, max_rows);
+}
+
 // q, k and z [rows, heads * Dk] (z: the decay's logits, before bias), v [rows, heads * P], bias [heads * Dk], state
-// [slots, heads, P, Dk], out [rows, heads * P]
+// [slots, heads, P, Dk], out [rows, heads * P].  `max_rows`: the most rows a sequence brings (0: unknown); `scratch`:
+// lq_gla_scan_workspace(...) floats, or null (then no segments).
 extern "C" int lq_gla_scan(const float* q, int ldq, const float* k, int ldk, const float* v, int ldv, const float* z, int ldz,
                            const float* bias, float* state, float* out, int ldo, int heads, int Dk, int P, float q_scale,
-                           float inv_tau, const int* seq_slot, const int* cu_rows, int batch, hipStream_t stream) {
+                           float inv_tau, const int* seq_slot, const int* cu_rows, int batch, int max_rows, float* scratch,
+                           long long scratch_floats, hipStream_t stream) {
   LQ_REQUIRE(heads > 0 && Dk > 0 && P > 0 && batch > 0, "gla_scan: bad sizes");
   LQ_REQUIRE(ldq >= heads * Dk && ldk >= heads * Dk && ldz >= heads * Dk && ldv >= heads * P && ldo >= heads * P,
              "gla_scan: a row stride is smaller than its row");
   LQ_REQUIRE(q && k && v && z && bias && state && out && seq_slot && cu_rows, "gla_scan: null pointer");
+  const long long need = scratch != nullptr ? gla_segment_floats(batch, heads, P, Dk, max_rows) : 0;
   ScanLaunch cfg;
   LQ_REQUIRE(scan_launch(Dk, P, (long long)batch * heads, cfg), "gla_scan: key size %d is too large", Dk);
+  LQ_REQUIRE(need <= scratch_floats, "gla_scan: %lld floats of scratch for a launch in segments, %lld given", need, scratch_floats);
   const int np = cfg.ln * cfg.slab;
   const size_t lds = 2 * (size_t)gla_tokens(np, cfg.threads, cfg.ln) * (3 * np + 2 * cfg.cols) * sizeof(float);
   LQ_REQUIRE(lds <= 64 * 1024, "gla_scan: key size %d is too large", Dk);
-  dim3 grid((unsigned)(batch * heads), lq_ceil_div(P, cfg.cols));
+  SegArgs sg = {1, 1, nullptr, nullptr};
+  if (need > 0) {
+    sg.nseg = SEG_COUNT;
+    sg.state = scratch;
+    sg.decay = scratch + (long long)batch * heads * SEG_COUNT * P * Dk;
+  }
+  dim3 grid((unsigned)(batch * heads), lq_ceil_div(P, cfg.cols), sg.nseg);
   ScanShape sh = {heads, heads, P, Dk, seq_slot, cu_rows};
 #define LQ_GLA(LN, SL, TH)                                                                                            \
   gla_scan_kernel<LN, SL, TH><<<grid, cfg.threads, lds, stream>>>(q, ldq, k, ldk, v, ldv, z, ldz, bias, state, out, ldo, \
-                                                                  sh, q_scale, inv_tau)
+                                                                  sh, q_scale, inv_tau, sg)
   LQ_SCAN_LANES(LQ_GLA)
-#undef LQ_GLA
   LQ_CHECK_LAUNCH("gla_scan");
+  if (sg.nseg > 1) {
+    gla_chain_kernel<<<dim3((unsigned)(batch * heads), (unsigned)lq_ceil_div64((long long)P * Dk, 256)), 256, 0, stream>>>(
+        state, heads, P, Dk, sg, seq_slot, cu_rows);
+    LQ_CHECK_LAUNCH("gla_scan(chain)");
+    sg.pass = 2;
+    LQ_SCAN_LANES(LQ_GLA)
+    LQ_CHECK_LAUNCH("gla_scan(second pass)");
+  }
+#undef LQ_GLA
   return 0;
 }

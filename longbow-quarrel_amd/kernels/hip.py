@@ -990,12 +990,23 @@ class HipKernels:
             if rc:
                 self._check(rc)
 
+    @query
+    def gla_scan_workspace(self, batch: int, heads: int, key_dim: int, value_dim: int, max_rows: int) -> int:
+        """Float32 entries of scratch with which `gla_scan` runs this launch in segments (0: it does not)."""
+        self.lib.lq_gla_scan_workspace.restype = c_longlong
+        return int(self.lib.lq_gla_scan_workspace(c_int(batch), c_int(heads), c_int(value_dim), c_int(key_dim),
+                                                  c_int(max_rows)))
+
     def gla_scan(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, z: torch.Tensor, bias: torch.Tensor,
                  state: torch.Tensor, out: torch.Tensor, heads: int, key_dim: int, value_dim: int, q_scale: float,
-                 inv_tau: float, seq_slot: torch.Tensor, cu_rows: torch.Tensor, batch: int) -> None:
+                 inv_tau: float, seq_slot: torch.Tensor, cu_rows: torch.Tensor, batch: int, max_rows: int = 0,
+                 workspace: Optional[torch.Tensor] = None) -> None:
         """Gated linear attention along every sequence of the step, token by token: with the decay a =
         sigmoid(z + bias)^inv_tau for every key channel, S <- diag(a) S + k v^T and out = S^T (q q_scale) per head;
-        state [slots, heads, value_dim, key_dim] is read and left at the step's end.  All float32."""
+        state [slots, heads, value_dim, key_dim] is read and left at the step's end.  All float32.  `max_rows` (the
+        most rows a sequence brings) and `workspace` (`gla_scan_workspace(...)` floats) let a launch of few long
+        sequences run in segments side by side (every segment from zero, the end states chained with the products
+        of the segments' decays, the segments again from their true starts)."""
         rows = q.shape[0]
         for t, what, cols in ((q, "q", heads * key_dim), (k, "k", heads * key_dim), (z, "z", heads * key_dim),
                               (v, "v", heads * value_dim), (out, "out", heads * value_dim)):
@@ -1008,12 +1019,15 @@ class HipKernels:
             raise KernelLibraryError("gla_scan: state must be dense [slots, heads, value_dim, key_dim]")
         self._i32(seq_slot, "seq_slot", batch)
         self._i32(cu_rows, "cu_rows", batch + 1)
+        if workspace is not None:
+            self._f32(workspace, "gla_scan: workspace", workspace.numel())
         ld = self._rows2d
         self._check(self.lib.lq_gla_scan(_ptr(q), c_int(ld(q, "q")), _ptr(k), c_int(ld(k, "k")), _ptr(v),
                                          c_int(ld(v, "v")), _ptr(z), c_int(ld(z, "z")), _ptr(bias), _ptr(state), _ptr(out),
                                          c_int(ld(out, "out")), c_int(heads), c_int(key_dim), c_int(value_dim),
                                          c_float(q_scale), c_float(inv_tau), _ptr(seq_slot), _ptr(cu_rows), c_int(batch),
-                                         self.stream))
+                                         c_int(max_rows if workspace is not None else 0), _ptr(workspace),
+                                         c_longlong(0 if workspace is None else workspace.numel()), self.stream))
 
     def moe_route(self, logits: torch.Tensor, route: torch.Tensor, top: int, renormalize: bool = False) -> None:
         """route[r, e] = sigmoid(logits[r, e]) for the `top` experts with the largest scores (the lower index on a

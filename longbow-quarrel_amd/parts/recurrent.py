@@ -346,9 +346,13 @@ class GatedLinearAttention(Mixer):
         z = ctx.ws.alloc((rows, qk), torch.float32)
         project(kn, ctx, low, self.w_a2, z)
         o = ctx.ws.alloc((rows, vw), torch.float32)
+        # a few long prompts: the kernel may cut them into segments that run side by side, given scratch
+        ask = getattr(kn, "gla_scan_workspace", None)
+        need = ask(ctx.batch, self.heads, self.key_dim, self.value_dim, ctx.max_new) if ask is not None else 0
+        more = dict(max_rows=ctx.max_new, workspace=ctx.ws.alloc((need,), torch.float32)) if need else {}
         kn.gla_scan(u[:, :qk], u[:, qk : 2 * qk], u[:, 2 * qk : 2 * qk + vw], z, self.a2_bias, cache.state, o,
                     self.heads, self.key_dim, self.value_dim, self.key_dim ** -0.5, 1.0 / self.tau,
-                    ctx.seq_slot, ctx.cu_rows, ctx.batch)
+                    ctx.seq_slot, ctx.cu_rows, ctx.batch, **more)
         normed = ctx.ws.alloc((rows, vw), ctx.dtype)
         kn.gated_rmsnorm(o, u[:, 2 * qk + vw : 2 * qk + 2 * vw], self.norm_w, self.eps, self.value_dim, normed,
                          gate_first=False)

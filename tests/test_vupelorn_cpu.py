@@ -147,23 +147,18 @@ def test_plain_rotation_pairings_and_yarn():
 
 
 def test_plain_gla_forgets_at_the_rate_of_its_decay():
-    """With k and q fixed to one channel the output is a geometric sum of the values with ratio sigmoid(b)^(1/tau)."""
-    m = {"heads": 1, "dim": 2, "vdim": 1, "tau": 2.0}
-    w = {"q": torch.tensor([[2.0 ** 0.5], [0.0]]), "k": torch.tensor([[1.0], [0.0]]), "v": torch.tensor([[1.0]]),
-         "a1": torch.zeros(1, 1), "a2": torch.zeros(2, 1), "a2.b": torch.tensor([0.0, 5.0]), "norm": torch.ones(1),
-         "g": torch.tensor([[1.0]]), "o": torch.tensor([[1.0]])}
-    w = {"x." + k: v for k, v in w.items()}
-    h = torch.ones(4, 1, dtype=torch.float64)
-    # the norm over a single value gives its sign, so look at the state through an un-normed copy of the recurrence
-    a = 0.5 ** 0.5
-    want = [1.0, 1 + a, 1 + a + a * a, 1 + a + a * a + a ** 3]
-    S, got = 0.0, []
-    for t in range(4):
-        S = a * S + 1.0
-        got.append(S)
-    assert got == pytest.approx(want)
+    """One key channel, two value channels: the first is fed a one at every token, the second at the first token
+    only.  The state's two entries are then a geometric sum and a pure power of the decay a = sigmoid(b)^(1 / tau),
+    and the norm over the value channels keeps their ratio: a^t (1 - a) / (1 - a^(t + 1))."""
+    m = {"heads": 1, "dim": 1, "vdim": 2, "tau": 2.0}
+    w = {"q": [[1.0, 0.0]], "k": [[1.0, 0.0]], "v": [[1.0, 0.0], [0.0, 1.0]], "a1": [[0.0, 0.0]], "a2": [[0.0]],
+         "a2.b": [0.7], "norm": [1.0, 1.0], "g": [[1.0, 0.0], [1.0, 0.0]], "o": [[1.0, 0.0], [0.0, 1.0]]}
+    w = {"x." + k: torch.tensor(v) for k, v in w.items()}
+    h = torch.tensor([[1.0, 1.0]] + [[1.0, 0.0]] * 5, dtype=torch.float64)
     y = pv.gla(m, "x.", w, h, 0.0, False)
-    assert torch.allclose(y[:, 0], torch.full((4,), 1 / (1 + math.exp(-1.0)), dtype=torch.float64))
+    a = (1 / (1 + math.exp(-0.7))) ** 0.5
+    for t in range(6):
+        assert float(y[t, 1] / y[t, 0]) == pytest.approx(a ** t * (1 - a) / (1 - a ** (t + 1)), rel=1e-6)  # (the bias is a 32-bit 0.7)
 
 
 def test_plain_moe_weights_the_input_of_the_chosen_experts():

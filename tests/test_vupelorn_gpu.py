@@ -91,6 +91,48 @@ def test_gated_linear_attention_scan_in_portions(kn, sizes):
     assert bool((state[[0, 2, 4]] == 7.0).all())  # nobody else's state was touched
 
 
+@pytest.mark.parametrize("sizes", [(2, 32, 24, 4.0), (1, 128, 256, 16.0), (3, 17, 9, 2.0)])
+def test_gated_linear_attention_scan_of_a_long_prompt_in_segments(kn, sizes):
+    """A long prompt beside a short one: the launch cuts the long one into segments that run side by side (from zero,
+    end states chained with the products of the decays, again from the true starts); the state it leaves is the
+    one that a token-by-token walk leaves, and a single token goes on from it."""
+    H, dk, dv, tau = sizes
+    n_long, n_short = 701, 30
+    g = torch.Generator().manual_seed(dk)
+    q, k, v = (torch.empty(n_long + n_short + 2, H * d).normal_(0, 1, generator=g) for d in (dk, dk, dv))
+    z = torch.empty(n_long + n_short + 2, H * dk).normal_(1, 2, generator=g)
+    bias = torch.empty(H * dk).normal_(2, 2, generator=g)
+    start = torch.empty(4, H, dv, dk).normal_(0, 1, generator=g)  # the sequences do not start from nothing
+
+    def plain(rows, S):
+        S = S.double().transpose(1, 2).clone()  # [head, key, value]
+        outs = []
+        for r in rows:
+            a = torch.sigmoid(z[r].double() + bias.double()).pow(1 / tau).reshape(H, dk)
+            S = a[:, :, None] * S + k[r].double().reshape(H, dk)[:, :, None] * v[r].double().reshape(H, dv)[:, None, :]
+            outs.append(torch.einsum("hkv,hk->hv", S, q[r].double().reshape(H, dk) * dk ** -0.5).reshape(-1))
+        return torch.stack(outs), S.transpose(1, 2)
+
+    need = kn.gla_scan_workspace(2, H, dk, dv, n_long)
+    assert need > 0
+    state = start.clone().to(DEV)
+    rows = n_long + n_short
+    out = torch.zeros(rows, H * dv, device=DEV)
+    kn.gla_scan(dev(q[:rows]), dev(k[:rows]), dev(v[:rows]), dev(z[:rows]), dev(bias), state, out, H, dk, dv, dk ** -0.5,
+                1 / tau, i32([2, 0]), i32([0, n_long, rows]), 2, max_rows=n_long,
+                workspace=torch.zeros(need, device=DEV))
+    want_long, s_long = plain(range(n_long), start[2])
+    want_short, s_short = plain(range(n_long, rows), start[0])
+    assert uc.err(out[:n_long].cpu(), want_long) < TOL_F32 and uc.err(out[n_long:].cpu(), want_short) < TOL_F32
+    assert uc.err(state[2].cpu(), s_long) < TOL_F32 and uc.err(state[0].cpu(), s_short) < TOL_F32
+    assert torch.equal(state[[1, 3]].cpu(), start[[1, 3]])
+    one = torch.zeros(2, H * dv, device=DEV)
+    kn.gla_scan(dev(q[rows:]), dev(k[rows:]), dev(v[rows:]), dev(z[rows:]), dev(bias), state, one, H, dk, dv, dk ** -0.5,
+                1 / tau, i32([2, 0]), i32([0, 1, 2]), 2)
+    assert uc.err(one[0].cpu(), plain([rows], s_long)[0][0]) < TOL_F32
+    assert uc.err(one[1].cpu(), plain([rows + 1], s_short)[0][0]) < TOL_F32
+
+
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 def test_norm_over_columns_rotation_and_the_norm_of_a_result(kn, dtype):
     rows, n = 9, 52
@@ -316,6 +358,11 @@ def test_a_slow_decay_keeps_old_tokens_in_the_state(cases):
     want = case.want(t)
     assert uc.err(case.run_cut(t, [260]), want) < TOL_F32
     assert uc.err(case.run_cut(t, [3, 64, 1, 2, 130]), want) < TOL_F32
+    # a prompt long enough for the scan in segments, then decoding from the state it left
+    t = uc.tokens(640, case.vocab, 32)
+    want = case.want(t)
+    assert uc.err(case.run_cut(t, [600]), want) < TOL_F32
+    assert uc.err(case.run_cut(t, [20, 580, 2]), want) < TOL_F32
 
 
 @pytest.mark.parametrize("name", ["a", "c"])
