@@ -215,6 +215,23 @@ def test_prompt_rows_sorted_by_expert(cases, name, monkeypatch):
     assert uc.err(case.run_cut(t, [50, 3, 30]), case.want(t)) < TOL
 
 
+@pytest.mark.parametrize("seed", [1, 2, 3, 4])
+def test_configurations_drawn_from_a_seed(cases, seed):
+    case = cases(seed)
+    assert lq.VupelornConfig.from_dict(case.cfg).to_dict() == case.cfg
+    t, u = uc.tokens(70, case.vocab, seed), uc.tokens(9, case.vocab, seed + 50)
+    assert uc.err(case.run_cut(t, [40, 2, 1, 20]), case.want(t)) < TOL
+    eng = case.eng
+    sa, sb = eng.new_sequence(), eng.new_sequence()
+    out = eng.step([StepEntry(sa, u[:8], range(8)), StepEntry(sb, t[:66], range(66))])
+    assert uc.err(out, torch.cat([case.want(u)[:8], case.want(t)[:66]])) < TOL
+    out = eng.step([StepEntry(sa, u[8:], [0]), StepEntry(sb, t[66:67], [0])])
+    assert uc.err(out, torch.stack([case.want(u)[8], case.want(t)[66]])) < TOL
+    eng.release(sa)
+    eng.release(sb)
+    case.assert_idle()
+
+
 def test_the_residual_stream_after_every_layer(cases):
     case = cases("a")
     got, want = case.layers(uc.tokens(37, case.vocab, 8))

@@ -310,6 +310,25 @@ def test_prompt_rows_sorted_by_expert(cases, name, dtype, monkeypatch):
         uc.assert_close_bf16(by_expert, case.want(t), case.noise(t))
 
 
+@pytest.mark.parametrize("seed", range(1, 13))
+def test_configurations_drawn_from_a_seed(cases, seed):
+    """Other sizes, head counts, ranks, layer orders, lenders of latents, experts and constants, in both dtypes."""
+    case = cases(seed)
+    t, u = uc.tokens(200, case.vocab, seed), uc.tokens(9, case.vocab, seed + 50)
+    assert uc.err(case.run_cut(t, [150, 2, 1, 20]), case.want(t)) < TOL_F32
+    eng = case.eng
+    sa, sb = eng.new_sequence(), eng.new_sequence()
+    out = eng.step([StepEntry(sa, u[:8], range(8)), StepEntry(sb, t[:130], range(130))])
+    assert uc.err(out, torch.cat([case.want(u)[:8], case.want(t)[:130]])) < TOL_F32
+    out = eng.step([StepEntry(sa, u[8:], [0]), StepEntry(sb, t[130:131], [0])])
+    assert uc.err(out, torch.stack([case.want(u)[8], case.want(t)[130]])) < TOL_F32
+    eng.release(sa)
+    eng.release(sb)
+    case.assert_idle()
+    case16 = cases(seed, "bfloat16")
+    uc.assert_close_bf16(case16.run_cut(t, [150, 2]), case16.want(t), case16.noise(t))
+
+
 def test_the_residual_stream_after_every_layer(cases):
     case = cases("a")
     got, want = case.layers(uc.tokens(37, case.vocab, 8))

@@ -86,6 +86,45 @@ CONFIGS = {"a": CFG_A, "b": CFG_B, "c": CFG_C, "gla": CFG_GLA, "latent": CFG_LAT
            "moe": CFG_MOE, "bigram": CFG_BIGRAM}
 
 
+def random_config(seed: int) -> dict:
+    """A configuration drawn from a seed: sizes, head counts, ranks, the order of the layers, which layers lend
+    their latent, experts and constants all vary; some sizes are multiples of 16, some of nothing."""
+    import random
+
+    rng = random.Random(seed)
+    even = lambda lo, hi: 2 * rng.randint(lo // 2, hi // 2)
+    width = rng.choice([40, 56, 64, 72, 100, 128, 136])
+    layers, latents = [], {}  # latents: layer index -> (kind, kv_rank, rot_dim, rot)
+    for i in range(rng.randint(2, 6)):
+        mlp = None if rng.random() < 0.2 else _moe(rng.randint(2, 6), 1, rng.choice([8, 12, 20, 32]), rng.choice([0.5, 2.0, 7.0]))
+        if mlp is not None:
+            mlp["router"]["top"] = rng.randint(1, mlp["router"]["experts"])
+        kind = rng.choice(["gla", "latent_attention", "latent_attention_2", "latent_attention_2"])
+        if kind == "gla":
+            layers.append(_gla(rng.randint(1, 4), rng.choice([8, 12, 16, 24, 40]), rng.choice([8, 12, 16, 36]),
+                               rng.choice([1.0, 4.0, 16.0]), rng.randint(1, 8), mlp))
+            continue
+        lend = [j for j, v in latents.items() if v[0] == kind]
+        if kind == "latent_attention_2" and lend and rng.random() < 0.5:
+            j = rng.choice(lend)
+            _, kv_rank, rot_dim, rot = latents[j]
+            layer = _latent(kind, rng.randint(1, 5), rng.choice([8, 16, 20]), rot_dim, rng.choice([8, 16, 28]), kv_rank,
+                            rng.choice([12, 16, 40]), rng.choice([0.1, 0.25]), rot["base"], mlp, kv_from=j)
+        else:
+            rot_dim = even(2, 24) if rng.random() < 0.5 else rng.choice([8, 16, 32])
+            scaling = None
+            if kind == "latent_attention":
+                scaling = {"factor": rng.choice([2.0, 4.0, 8.0]), "original": rng.choice([16, 64, 2048]),
+                           "fast": rng.choice([8.0, 32.0]), "slow": rng.choice([1.0, 2.0])}
+            layer = _latent(kind, rng.randint(1, 5), rng.choice([8, 16, 20, 32]), rot_dim, rng.choice([8, 16, 28]),
+                            rng.choice([8, 16, 24, 40, 48]), rng.choice([12, 16, 40]), rng.choice([0.1, 0.25]),
+                            rng.choice([100.0, 10000.0, 250000.0]), mlp, scaling=scaling)
+            latents[i] = (kind, layer["mixer"]["kv_rank"], rot_dim, layer["mixer"]["rot"])
+        layers.append(layer)
+    bigram = None if rng.random() < 0.3 else (rng.randint(3, 300), rng.randint(1, 99), rng.randint(1, 99))
+    return _config(rng.randint(30, 300), width, rng.choice([1e-6, 1e-5]), layers, bigram)
+
+
 def make_weights(cfg: dict, seed: int, sharp: float = 1.0, memory: float = 0.0) -> Dict[str, torch.Tensor]:
     """Random weights whose values bfloat16 holds exactly (both run dtypes then see the same model), with spreads
     that make every constant matter.  `sharp` scales the queries' and the latents' projections so that attention
@@ -140,7 +179,7 @@ class Case:
 
     def __init__(self, tmp_path, name: str, load, dtype: str = "float32", seed: int = 3, sharp: float = 1.0,
                  memory: float = 0.0, max_tokens: int = 2048, rounding: bool = False) -> None:
-        self.cfg = copy.deepcopy(CONFIGS[name])
+        self.cfg = copy.deepcopy(CONFIGS[name] if isinstance(name, str) else random_config(name))
         self.weights = make_weights(self.cfg, seed, sharp, memory)
         self.folder = write_folder(tmp_path, self.cfg, self.weights, f"{name}_{seed}_{sharp}_{memory}")
         self.eng = load(self.folder, dtype, max_tokens)
