@@ -45,12 +45,12 @@ def _mixer(cfg: VupelornConfig, layer: VupelornLayer, i: int) -> PartSpec:
 def vupelorn_spec(cfg: VupelornConfig) -> ModelSpec:
     blocks, schedule = [], []
     for i, layer in enumerate(cfg.layers):
-        ffn = ffn_norm = None
+        ffn = None
+        ffn_norm = PartSpec("rmsnorm", {"width": cfg.width, "eps": cfg.norm_eps, "name": f"l{i}.norm2"})
         if layer.mlp is not None:
             e = layer.mlp
             ffn = PartSpec("moe", {"width": cfg.width, "experts": e.experts, "top": e.top, "inner": e.ff,
                                    "limit": e.limit, "prefix": f"l{i}.mlp", "weight_input": True})
-            ffn_norm = PartSpec("rmsnorm", {"width": cfg.width, "eps": cfg.norm_eps, "name": f"l{i}.norm2"})
         blocks.append(PartSpec("output_norm", {
             "mixer": _mixer(cfg, layer, i),
             "mixer_norm": PartSpec("rmsnorm", {"width": cfg.width, "eps": cfg.norm_eps, "name": f"l{i}.norm1"}),

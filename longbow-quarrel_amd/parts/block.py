@@ -5,6 +5,7 @@ the norm kernel that follows it, or, for the few rows of a decoding step, on the
 produced it, which then also leaves the statistics for the norm that the next projection folds in."""
 from __future__ import annotations
 
+import dataclasses
 from typing import List, Mapping, Optional
 
 import torch
@@ -175,6 +176,8 @@ class OutputNormBlock(Block):
         self.ffn_norm = build_part(NORMS, ffn_norm) if feed_forward is not None else None
         if feed_forward is not None and ffn_norm is None:
             raise ValueError("a feed-forward needs the norm of its result")
+        # the norm of a feed-forward that is not there: a file may hold its weight all the same; it is not used
+        self.idle_norm = build_part(NORMS, ffn_norm) if feed_forward is None and ffn_norm is not None else None
         for norm in (self.mixer_norm, self.ffn_norm):
             if norm is not None and not getattr(norm, "deferrable", False):
                 raise ValueError("the norms on the sublayers' results must be RMS norms")
@@ -187,7 +190,10 @@ class OutputNormBlock(Block):
         return tuple(p for p in (self.mixer, self.mixer_norm, self.ffn, self.ffn_norm) if p is not None)
 
     def tensor_specs(self) -> List[TensorSpec]:
-        return [s for p in self.parts() for s in p.tensor_specs()]
+        specs = [s for p in self.parts() for s in p.tensor_specs()]
+        if self.idle_norm is not None:
+            specs += [dataclasses.replace(s, optional=True) for s in self.idle_norm.tensor_specs()]
+        return specs
 
     def bind(self, tensors: Mapping[str, torch.Tensor], env: BuildEnv) -> None:
         super().bind(tensors, env)

@@ -36,6 +36,8 @@ def random_tensors(specs: Sequence[TensorSpec], seed: int, dtype: torch.dtype, s
     device = torch.device(device or "cpu")
     out: Dict[str, torch.Tensor] = {}
     for s in specs:
+        if s.optional:  # what a file may leave out, random weights leave out
+            continue
         gen = torch.Generator(device=device)
         gen.manual_seed(_tensor_seed(seed, s.name))
         if s.kind == TABLE:

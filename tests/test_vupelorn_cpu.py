@@ -49,7 +49,9 @@ def test_configuration_reads_every_size_and_writes_the_same_keys_back():
     assert {"bigram", "l0.mix.dkv.norm", "l1.mix.a2.b", "l2.mix.dkv", "l3.mix.uk", "l0.mlp.e4.down", "l0.mlp.router",
             "l4.norm2", "final.norm"} <= names
     assert "l3.mix.dkv" not in names and "l3.mix.dkv.norm" not in names  # the layer reads another's latent
-    assert "l1.norm2" not in names and not any(n.startswith("l1.mlp") for n in names)  # no feed-forward, no norm of it
+    assert not any(n.startswith("l1.mlp") for n in names)  # no feed-forward
+    # the norm of a feed-forward that is not there may be in a file or not
+    assert [s.optional for s in model.tensor_specs() if s.name == "l1.norm2"] == [True]
     assert "head" not in names  # the head is the embedding
     needs = model.cache_needs()
     assert set(needs) == {EMBEDDING_RUN, 0, 1, 2, 4}
@@ -99,6 +101,18 @@ def test_a_size_that_no_key_gives_comes_from_the_file(tmp_path):
     with pytest.raises(lq.ConfigError) as e:
         lq.random_engine(lq.VupelornConfig.from_dict(cfg), 1, device="cpu", kernels=CpuKernels())
     assert "decay" in str(e.value)
+
+
+def test_the_norm_of_an_absent_feed_forward_may_be_in_the_file(tmp_path):
+    cfg = copy.deepcopy(uc.CFG_GLA)
+    weights = uc.make_weights(cfg, 5)
+    assert "l0.norm2" not in weights
+    t = uc.tokens(12, cfg["vocab"], 1)
+    got = []
+    for name, extra in (("without", {}), ("with", {"l0.norm2": torch.full((cfg["width"],), 3.0)})):
+        eng = load(uc.write_folder(tmp_path, cfg, {**weights, **extra}, name), "float32", 256)
+        got.append(eng.step([StepEntry(eng.new_sequence(), t, range(12))]))
+    assert torch.equal(got[0], got[1]) and uc.err(got[0], pv.forward(cfg, weights, t)) < TOL
 
 
 def test_missing_and_unexpected_tensors_are_named(tmp_path):

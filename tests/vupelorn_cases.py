@@ -137,6 +137,8 @@ def make_weights(cfg: dict, seed: int, sharp: float = 1.0, memory: float = 0.0) 
     g = torch.Generator().manual_seed(seed)
     out = {}
     for s in DecoderModel(spec_from_config(config)).tensor_specs():
+        if s.optional:  # (the norm of a feed-forward that is not there)
+            continue
         n, shape = s.name, tuple(s.shape)
         leaf = n.split(".")[-1]
         normal = lambda std, mean=0.0: torch.empty(shape).normal_(mean, std, generator=g)
