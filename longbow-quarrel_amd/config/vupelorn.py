@@ -87,7 +87,8 @@ class Rotary:
     scaling: Optional[RotaryScaling]
 
     @classmethod
-    def from_dict(cls, d, where):
+    def from_dict(cls, d, where, whole: Optional[int] = None):
+        """`whole`: the size of the rotated part, which `dims` defaults to."""
         sc = d.get("scaling") if isinstance(d, dict) else None
         scaling = None
         if sc is not None:
@@ -96,7 +97,8 @@ class Rotary:
                                     _get(sc, "fast", w, float), _get(sc, "slow", w, float))
             if not scaling.factor > 0 or not scaling.original > 0 or not scaling.fast > 0 or not scaling.slow > 0:
                 raise ConfigError(f"config.json: '{w}' needs positive factor, original, fast and slow")
-        c = cls(_get(d, "base", where, float), _get(d, "dims", where, least=2), scaling)
+        c = cls(_get(d, "base", where, float),
+                _get(d, "dims", where, least=2, default=_REQUIRED if whole is None else whole), scaling)
         if c.dims % 2 or not c.base > 0:
             raise ConfigError(f"config.json: '{where}.dims' must be even and '{where}.base' positive")
         return c
@@ -123,10 +125,12 @@ class LatentMixer:
     @classmethod
     def from_dict(cls, d, where):
         dim = _get(d, "dim", where, least=1)
-        c = cls(_get(d, "heads", where, least=1), dim, _get(d, "rot_dim", where, least=2),
+        rot_dim = _get(d, "rot_dim", where, least=2)
+        c = cls(_get(d, "heads", where, least=1), dim, rot_dim,
                 _get(d, "vdim", where, least=1, default=dim), _get(d, "kv_rank", where, least=1),
                 _get(d, "q_rank", where, least=1), _get(d, "scale", where, float),
-                Rotary.from_dict(d.get("rot"), where + ".rot"), _get(d, "kv_from", where, least=0, default=None))
+                Rotary.from_dict(d.get("rot"), where + ".rot", whole=rot_dim),
+                _get(d, "kv_from", where, least=0, default=None))
         if c.rot.dims > c.rot_dim:
             raise ConfigError(f"config.json: '{where}.rot.dims' ({c.rot.dims}) is more than rot_dim ({c.rot_dim})")
         return c

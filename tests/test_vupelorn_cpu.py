@@ -86,6 +86,14 @@ def test_configuration_errors_name_their_key(key, value, text):
     assert text in str(e.value)
 
 
+def test_keys_that_a_configuration_leaves_out_take_the_sizes_they_follow():
+    cfg = copy.deepcopy(uc.CFG_LATENT2)
+    m = cfg["layers"][0]["mixer"]
+    del m["rot"]["dims"], m["vdim"]
+    got = lq.VupelornConfig.from_dict(cfg).layers[0].latent
+    assert got.rot.dims == m["rot_dim"] and got.vdim == m["dim"]
+
+
 def test_a_size_that_no_key_gives_comes_from_the_file(tmp_path):
     """The rank of the decay's bottleneck is the shape of its first matrix; without a file it must be stated."""
     cfg = copy.deepcopy(uc.CFG_GLA)
