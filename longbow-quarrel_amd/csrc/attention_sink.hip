@@ -36,6 +36,11 @@ struct SinkArgs {
   int bt_stride, BS;
   float scale;
   int window, keep_first, sink;
+  // single tokens of a bfloat16 run may share a tile's keys out over `ksplit` workgroups (blockIdx.z): each takes
+  // the rounds of SPLIT chunks whose number is its own modulo ksplit and leaves its partial result in `part`,
+  // which a second launch merges in the order of the workgroups
+  int ksplit;
+  float* part;
 };
 
 constexpr int MAX_KD = 256;
@@ -86,7 +91,7 @@ __global__ __launch_bounds__(64 * SPLIT) void sink_tiles_kernel(const T* __restr
   __syncthreads();
 
   // the sink is one more key of score 0 without a value: the first wavefront starts from it
-  const bool with_sink = a.sink && wave == 0;
+  const bool with_sink = a.sink && wave == 0 && blockIdx.z == 0;
   float m = with_sink ? 0.f : -INFINITY, l = with_sink ? 1.f : 0.f;
   f32x4 o[HSV];  // o[dt][e]: row 4 g + e of the tile, value dimension 16 dt + c
 #pragma unroll
@@ -110,7 +115,7 @@ __global__ __launch_bounds__(64 * SPLIT) void sink_tiles_kernel(const T* __restr
     const int kept_end = min(a.keep_first, wstart);  // kept keys that lie below that chunk
     int t0 = kept_end > 0 ? 0 : wstart;
     while (t0 <= pos_max) {
-      if (((t0 >> 6) & (SPLIT - 1)) == wave) {
+      if (((t0 >> 6) & (SPLIT - 1)) == wave && (a.ksplit == 1 || (t0 >> 8) % a.ksplit == (int)blockIdx.z)) {
         f32x4 st[4];  // st[kt][e]: score of key t0 + 16 kt + 4 g + e for row c
 #pragma unroll
         for (int kt = 0; kt < 4; ++kt) {
@@ -217,6 +222,13 @@ __global__ __launch_bounds__(64 * SPLIT) void sink_tiles_kernel(const T* __restr
       for (int dt = 0; dt < HSV; ++dt) o[dt][e] = o[dt][e] * fa + part[(dt * 64 + lane) * 4 + e] * fb;
     }
   }
+  if (a.ksplit > 1) {  // this workgroup's share of the keys: the merge launch finishes the tile
+    float* mine_part = a.part + (((long long)blockIdx.y * gridDim.x + blockIdx.x) * a.ksplit + blockIdx.z) * PART;
+#pragma unroll
+    for (int dt = 0; dt < HSV; ++dt) *(f32x4*)(mine_part + (dt * 64 + lane) * 4) = o[dt];
+    if (g == 0) mine_part[64 * HSV * 4 + c] = m, mine_part[64 * HSV * 4 + 16 + c] = l;
+    return;
+  }
   float inv4[4];
   const float inv = 1.0f / l;
 #pragma unroll
@@ -224,6 +236,56 @@ __global__ __launch_bounds__(64 * SPLIT) void sink_tiles_kernel(const T* __restr
 #pragma unroll
   for (int e = 0; e < 4; ++e) {
     const int tr = 4 * g + e, row = tr / GH, hh = hbase + tr % GH;  // tile row -> step row and head
+    if (row < n_rows) {
+      float f = inv4[e];
+      if (gate != nullptr) f /= 1.f + expf(-to_f32(gate[(long long)(r0 + row) * a.ldg + hh]));
+      T* orow = out + (long long)(r0 + row) * a.ldo + hh * (HSV * 16) + c;
+#pragma unroll
+      for (int dt = 0; dt < HSV; ++dt) orow[dt * 16] = from_f32<T>(o[dt][e] * f);
+    }
+  }
+}
+
+// The partial results of the `ksplit` workgroups of a tile, merged in their order (as the wavefronts of a workgroup
+// are), then the division by the sum, the gate and the store.  One wavefront a tile.
+template <typename T, int HSV>
+__global__ __launch_bounds__(64) void sink_merge_kernel(T* __restrict__ out, const T* __restrict__ gate, SinkArgs a) {
+  constexpr int PART = 64 * (HSV * 4) + 32;
+  const int lane = threadIdx.x, c = lane & 15, g = lane >> 4;
+  const int GH = a.heads_per_tile, hbase = blockIdx.y * GH, r0 = blockIdx.x * a.rows_per_tile;
+  const int n_rows = min(a.rows_per_tile, a.rows - r0);
+  const float* part = a.part + ((long long)blockIdx.y * gridDim.x + blockIdx.x) * a.ksplit * PART;
+  f32x4 o[HSV];
+#pragma unroll
+  for (int dt = 0; dt < HSV; ++dt) o[dt] = *(const f32x4*)(part + (dt * 64 + lane) * 4);
+  float m = part[64 * HSV * 4 + c], l = part[64 * HSV * 4 + 16 + c];
+  float m4[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) m4[e] = part[64 * HSV * 4 + 4 * g + e];
+  for (int w = 1; w < a.ksplit; ++w) {
+    part += PART;
+    const float mw = part[64 * HSV * 4 + c], lw = part[64 * HSV * 4 + 16 + c];
+    const float m_new = fmaxf(m, mw);
+    const bool none = m_new == -INFINITY;
+    l = none ? 0.f : l * expf(m - m_new) + lw * expf(mw - m_new);
+    m = m_new;
+#pragma unroll
+    for (int e = 0; e < 4; ++e) {
+      const float mo = part[64 * HSV * 4 + 4 * g + e];
+      const float mn = fmaxf(m4[e], mo);
+      const float fa = mn == -INFINITY ? 0.f : expf(m4[e] - mn), fb = mn == -INFINITY ? 0.f : expf(mo - mn);
+      m4[e] = mn;
+#pragma unroll
+      for (int dt = 0; dt < HSV; ++dt) o[dt][e] = o[dt][e] * fa + part[(dt * 64 + lane) * 4 + e] * fb;
+    }
+  }
+  const float inv = 1.0f / l;
+  float inv4[4];
+#pragma unroll
+  for (int e = 0; e < 4; ++e) inv4[e] = __shfl(inv, 4 * g + e, 64);
+#pragma unroll
+  for (int e = 0; e < 4; ++e) {
+    const int tr = 4 * g + e, row = tr / GH, hh = hbase + tr % GH;
     if (row < n_rows) {
       float f = inv4[e];
       if (gate != nullptr) f /= 1.f + expf(-to_f32(gate[(long long)(r0 + row) * a.ldg + hh]));
@@ -326,23 +388,63 @@ __global__ __launch_bounds__(256) void kv_store_kernel(const T* __restrict__ k, 
   }
 }
 
+// How a launch is cut into tiles, and over how many workgroups a tile's keys are shared out: one decision for the
+// query about scratch and for the launch.  Keys are shared out for single tokens of a bfloat16 run only (a float32
+// row's sums keep the one order that depends on its position alone), where the tiles alone leave most of the chip
+// idle and a wavefront would walk several rounds of chunks.
+struct TileShape {
+  bool tiles;
+  int heads_per_tile, rows_per_tile, grid_x, grid_y, ksplit;
+  long long part_floats;  // scratch for the partial results (0: no sharing out)
+};
+
+TileShape tile_shape(int el, int rows, int batch, int nh, int nkv, int KD, int VD, int BS, int window, int keep_first,
+                     int max_len) {
+  TileShape t = {false, 1, 1, 0, 0, 1, 0};
+  if (KD % 16 != 0 || VD % 16 != 0 || KD > MAX_KD || VD > 256 || BS % 16 != 0) return t;
+  const int hsv = VD / 16;
+  if (!(hsv <= 10 || hsv == 12 || hsv == 16)) return t;
+  t.tiles = true;
+  // the query heads of a kv head share a tile where their number is a power of two (or a multiple of 16)
+  const int group = nh / nkv;
+  t.heads_per_tile = group % 16 == 0 ? 16 : (group & (group - 1)) == 0 ? group : 1;
+  t.rows_per_tile = rows == batch ? 1 : 16 / t.heads_per_tile;  // single tokens: a tile a row of the step
+  t.grid_x = lq_ceil_div(rows, t.rows_per_tile), t.grid_y = nh / t.heads_per_tile;
+  if (el == 2 && rows == batch && max_len > 0) {
+    const int keys = window > 0 ? (max_len < window + keep_first + 128 ? max_len : window + keep_first + 128) : max_len;
+    const int rounds = lq_ceil_div(lq_ceil_div(keys, 64), SPLIT);
+    const long long tiles = (long long)t.grid_x * t.grid_y;
+    long long k = 2ll * lq_compute_units() / (tiles > 0 ? tiles : 1);
+    if (k > rounds) k = rounds;
+    if (k > 8) k = 8;
+    if (k >= 2) {
+      t.ksplit = (int)k;
+      t.part_floats = tiles * k * (64ll * hsv * 4 + 32);
+    }
+  }
+  return t;
+}
+
 template <typename T>
 bool launch_tiles(const void* q, void* out, const void* gate, const void* kcache, const void* vcache, const SinkArgs& a,
-                  int batch, hipStream_t stream) {
+                  int batch, int max_len, float* part, long long part_floats, hipStream_t stream) {
   const int el = (int)sizeof(T);
-  if (a.KD % 16 != 0 || a.VD % 16 != 0 || a.KD > MAX_KD || a.VD > 256 || a.BS % 16 != 0 || a.ldq % 4 != 0 ||
-      ((uintptr_t)q % (4 * el)) != 0 || ((uintptr_t)kcache % (4 * el)) != 0 || ((uintptr_t)vcache % (4 * el)) != 0)
+  if (a.ldq % 4 != 0 || ((uintptr_t)q % (4 * el)) != 0 || ((uintptr_t)kcache % (4 * el)) != 0 ||
+      ((uintptr_t)vcache % (4 * el)) != 0)
     return false;
+  const TileShape t = tile_shape(el, a.rows, batch, a.nh, a.nkv, a.KD, a.VD, a.BS, a.window, a.keep_first,
+                                 part != nullptr ? max_len : 0);
+  if (!t.tiles) return false;
   SinkArgs b = a;
-  // the query heads of a kv head share a tile where their number is a power of two (or a multiple of 16)
-  const int group = a.nh / a.nkv;
-  b.heads_per_tile = group % 16 == 0 ? 16 : (group & (group - 1)) == 0 ? group : 1;
-  b.rows_per_tile = a.rows == batch ? 1 : 16 / b.heads_per_tile;  // single tokens: a tile a row of the step
-  dim3 grid(lq_ceil_div(a.rows, b.rows_per_tile), a.nh / b.heads_per_tile);
+  b.heads_per_tile = t.heads_per_tile, b.rows_per_tile = t.rows_per_tile;
+  b.ksplit = t.part_floats > 0 && t.part_floats <= part_floats ? t.ksplit : 1;
+  b.part = part;
+  dim3 grid(t.grid_x, t.grid_y, b.ksplit);
 #define LQ_SINK(HSV)                                                                                                  \
   case HSV:                                                                                                           \
     sink_tiles_kernel<T, HSV><<<grid, 64 * SPLIT, 0, stream>>>((const T*)q, (T*)out, (const T*)gate, (const T*)kcache,        \
                                                        (const T*)vcache, b);                                          \
+    if (b.ksplit > 1) sink_merge_kernel<T, HSV><<<dim3(t.grid_x, t.grid_y), 64, 0, stream>>>((T*)out, (const T*)gate, b);   \
     return true;
   switch (a.VD / 16) {
     LQ_SINK(1) LQ_SINK(2) LQ_SINK(3) LQ_SINK(4) LQ_SINK(5) LQ_SINK(6) LQ_SINK(7) LQ_SINK(8) LQ_SINK(9) LQ_SINK(10)
@@ -373,12 +475,21 @@ extern "C" int lq_kv_store(const void* k, int ldk, const void* v, int ldv, int d
   return 0;
 }
 
-// `gate`: null, or [rows, nh] logits (stride ldg) in the dtype of q.  `rows == batch` means single tokens.
+// Float32 entries of scratch with which a launch of single tokens shares its keys out over several workgroups a tile
+// (0: it does not).  `max_len`: an upper bound of the sequences' lengths.
+extern "C" long long lq_sink_attention_workspace(int dtype, int rows, int batch, int nh, int nkv, int KD, int VD,
+                                                 int block_size, int window, int keep_first, int max_len) {
+  if (rows <= 0 || batch <= 0 || nh <= 0 || nkv <= 0 || nh % nkv != 0 || block_size <= 0) return 0;
+  return tile_shape(dtype == LQ_BF16 ? 2 : 4, rows, batch, nh, nkv, KD, VD, block_size, window, keep_first, max_len).part_floats;
+}
+
+// `gate`: null, or [rows, nh] logits (stride ldg) in the dtype of q.  `rows == batch` means single tokens.  `part`:
+// lq_sink_attention_workspace(...) floats for `max_len`, or null.
 extern "C" int lq_sink_attention(const void* q, int ldq, void* out, int ldo, const void* gate, int ldg, int dtype, int rows,
                                  int batch, int nh, int nkv, int KD, int VD, const int* row_pos, const int* row_seq,
                                  const int* seq_slot, const int* block_table, int bt_stride, const void* kcache,
                                  const void* vcache, int block_size, float scale, int window, int keep_first, int sink,
-                                 int force_rows, hipStream_t stream) {
+                                 int force_rows, int max_len, float* part, long long part_floats, hipStream_t stream) {
   LQ_REQUIRE(rows > 0 && batch > 0 && rows >= batch, "sink_attention: rows %d and sequences %d", rows, batch);
   LQ_REQUIRE(nh > 0 && nkv > 0 && nh % nkv == 0 && nh <= 65535, "sink_attention: %d heads over %d kv heads", nh, nkv);
   LQ_REQUIRE(KD > 0 && VD > 0 && KD <= MAX_DIM && VD <= MAX_DIM, "sink_attention: key size %d, value size %d", KD, VD);
@@ -390,9 +501,11 @@ extern "C" int lq_sink_attention(const void* q, int ldq, void* out, int ldo, con
   a.ldq = ldq, a.ldo = ldo, a.ldg = ldg, a.rows = rows, a.rows_per_tile = 1, a.heads_per_tile = 1, a.nh = nh, a.nkv = nkv, a.KD = KD, a.VD = VD;
   a.row_pos = row_pos, a.row_seq = row_seq, a.seq_slot = seq_slot, a.block_table = block_table;
   a.bt_stride = bt_stride, a.BS = block_size, a.scale = scale, a.window = window, a.keep_first = keep_first, a.sink = sink;
+  a.ksplit = 1, a.part = nullptr;
   if (!force_rows) {
-    const bool done = dtype == LQ_F32 ? launch_tiles<float>(q, out, gate, kcache, vcache, a, batch, stream)
-                                      : launch_tiles<bf16_t>(q, out, gate, kcache, vcache, a, batch, stream);
+    const bool done = dtype == LQ_F32
+                          ? launch_tiles<float>(q, out, gate, kcache, vcache, a, batch, max_len, part, part_floats, stream)
+                          : launch_tiles<bf16_t>(q, out, gate, kcache, vcache, a, batch, max_len, part, part_floats, stream);
     if (done) {
       LQ_CHECK_LAUNCH("sink_attention(tiles)");
       return 0;

@@ -696,15 +696,31 @@ class HipKernels:
         if seq_slot.dtype != torch.int32 or block_table.dtype != torch.int32 or block_table.dim() != 2:
             raise KernelLibraryError(f"{what}: seq_slot and block_table must be int32 (table 2-D)")
 
+    @query
+    def sink_attention_workspace(self, dtype: torch.dtype, rows: int, batch: int, heads: int, kv_heads: int, key_dim: int,
+                                 value_dim: int, block_size: int, window: int, keep_first: int, max_len: int) -> int:
+        """Float32 entries of scratch with which `sink_attention` shares the keys of a launch of single tokens out
+        over several workgroups a tile (0: it does not); `max_len`: an upper bound of the lengths."""
+        if dtype not in _DTYPE_CODE:
+            return 0
+        self.lib.lq_sink_attention_workspace.restype = c_longlong
+        return int(self.lib.lq_sink_attention_workspace(c_int(_DTYPE_CODE[dtype]), c_int(rows), c_int(batch), c_int(heads),
+                                                        c_int(kv_heads), c_int(key_dim), c_int(value_dim),
+                                                        c_int(block_size), c_int(window), c_int(keep_first),
+                                                        c_int(max_len)))
+
     def sink_attention(self, q: torch.Tensor, out: torch.Tensor, heads: int, kv_heads: int, key_dim: int,
                        value_dim: int, row_pos: torch.Tensor, row_seq: torch.Tensor, seq_slot: torch.Tensor,
                        block_table: torch.Tensor, kcache: torch.Tensor, vcache: torch.Tensor, block_size: int,
                        scale: float, window: int = 0, keep_first: int = 0, sink: bool = True,
-                       gate: Optional[torch.Tensor] = None, decode: bool = False) -> None:
+                       gate: Optional[torch.Tensor] = None, decode: bool = False, max_len: int = 0,
+                       workspace: Optional[torch.Tensor] = None) -> None:
         """Attention of the step's rows over their slots' cached keys: row at position p sees t <= p with
         p - t < window (0: all) or t < keep_first; with `sink` the softmax's denominator has one more term e^0;
         `gate` [rows, heads]: every head's result times the sigmoid of its entry.  Scores and probabilities
-        are 32-bit.  out [rows, heads * value_dim] in the dtype of q and the cache."""
+        are 32-bit.  out [rows, heads * value_dim] in the dtype of q and the cache.  `max_len` (an upper bound of the
+        lengths) and `workspace` (`sink_attention_workspace(...)` floats) let a launch of single tokens share a tile's
+        keys out over several workgroups (bfloat16 runs only)."""
         self._dev(q, out, gate, row_pos, row_seq, seq_slot, block_table, kcache, vcache)
         rows, batch = q.shape[0], seq_slot.numel()
         self._i32(row_pos, "row_pos", rows)
@@ -717,13 +733,16 @@ class HipKernels:
             raise KernelLibraryError("sink_attention: the gate is [rows, heads] in the dtype of q")
         if decode and rows != batch:
             raise KernelLibraryError("sink_attention: decode means one row per sequence")
+        if workspace is not None:
+            self._f32(workspace, "sink_attention: workspace", workspace.numel())
         self._check(self.lib.lq_sink_attention(
             _ptr(q), c_int(self._rows2d(q, "q")), _ptr(out), c_int(self._rows2d(out, "out")), _ptr(gate),
             c_int(0 if gate is None else self._rows2d(gate, "gate")), c_int(_code(q)), c_int(rows), c_int(batch),
             c_int(heads), c_int(kv_heads), c_int(key_dim), c_int(value_dim), _ptr(row_pos), _ptr(row_seq),
             _ptr(seq_slot), _ptr(block_table), c_int(int(block_table.stride(0))), _ptr(kcache), _ptr(vcache),
             c_int(block_size), c_float(scale), c_int(window), c_int(keep_first), c_int(1 if sink else 0),
-            c_int(1 if self.force_generic else 0), self.stream))
+            c_int(1 if self.force_generic else 0), c_int(max_len if workspace is not None else 0), _ptr(workspace),
+            c_longlong(0 if workspace is None else workspace.numel()), self.stream))
 
     # ------------------------------------------------------------------ recurrent mixers and what surrounds them
     _ACTIVATIONS = {"none": 0, "silu": 1, "relu": 2, "gelu_tanh": 3}

@@ -29,6 +29,7 @@ import torch
 from .base import (MIXERS, VECTOR32, BuildEnv, KVNeed, LayerCache, Mixer, StepContext, TensorSpec, product_weight,
                    project)
 from .rope import rotary_frequencies, rotary_magnitude
+from .sink_attention import split_scratch
 
 
 def _round8(n: int) -> int:
@@ -131,7 +132,7 @@ class LatentAttention(Mixer):
         mean = ctx.ws.alloc((rows, H * r), ctx.dtype)  # every head's weighted mean of latents
         kn.sink_attention(q, mean, H, 1, kd, r, ctx.row_pos, ctx.row_seq, ctx.seq_slot, cache.block_table, cache.k,
                           cache.v, cache.block_size, self.scale, window=0, keep_first=0, sink=False, gate=None,
-                          decode=ctx.decode)
+                          decode=ctx.decode, **split_scratch(ctx, q.dtype, H, 1, kd, r, cache.block_size, 0, 0))
         att = ctx.ws.alloc((rows, H * self.value_dim), ctx.dtype)
         kn.linear_heads(mean, self.w_uv, att, H, self.value_dim)
         if out is None:

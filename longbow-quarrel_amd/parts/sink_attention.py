@@ -22,6 +22,17 @@ from .base import (MIXERS, POSITION_ENCODINGS, BuildEnv, KVNeed, LayerCache, Mix
                    TensorSpec, build_part, product_weight, project)
 
 
+def split_scratch(ctx: StepContext, dtype, heads: int, kv_heads: int, key_dim: int, value_dim: int, block_size: int,
+                  window: int, keep_first: int) -> Dict[str, object]:
+    """The keywords with which `sink_attention` may share a decoding step's keys out over several workgroups a tile:
+    the step's bound of the lengths and the scratch that the kernel object asks for (nothing where it asks for none)."""
+    ask = getattr(ctx.kernels, "sink_attention_workspace", None)
+    if ask is None or not ctx.decode:
+        return {}
+    need = ask(dtype, ctx.rows, ctx.batch, heads, kv_heads, key_dim, value_dim, block_size, window, keep_first, ctx.max_len)
+    return dict(max_len=ctx.max_len, workspace=ctx.ws.alloc((need,), torch.float32)) if need else {}
+
+
 @MIXERS.register("sink_window_attention")
 class SinkWindowAttention(Mixer):
     takes_out = True
@@ -101,7 +112,9 @@ class SinkWindowAttention(Mixer):
         kn.sink_attention(q, att, self.heads, self.kv_heads, self.key_dim, self.value_dim, ctx.row_pos, ctx.row_seq,
                           ctx.seq_slot, cache.block_table, cache.k, cache.v, cache.block_size, self.scale,
                           window=self.window, keep_first=self.keep_first, sink=self.sink, gate=gate,
-                          decode=ctx.decode)
+                          decode=ctx.decode, **split_scratch(ctx, q.dtype, self.heads, self.kv_heads, self.key_dim,
+                                                             self.value_dim, cache.block_size, self.window,
+                                                             self.keep_first))
         if out is None:
             out = ctx.ws.alloc((rows, self.width), torch.float32)
         project(kn, ctx, att, self.w_o, out)

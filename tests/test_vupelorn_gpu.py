@@ -359,6 +359,35 @@ def test_bfloat16_whole_in_portions_and_in_batches(cases, name):
     case.assert_idle()
 
 
+def test_bfloat16_decoding_over_contexts_whose_keys_are_shared_out(cases, kn):
+    """Single tokens over several hundred cached rows: a tile's keys go to several workgroups and a second launch
+    merges them; against the same rows as parts of a prompt (one workgroup a tile) and against the plain
+    implementation."""
+    case = cases("c", "bfloat16")
+    m = case.cfg["layers"][0]["mixer"]
+    assert kn.sink_attention_workspace(torch.bfloat16, 2, 2, m["heads"], 1, m["kv_rank"] + m["rot_dim"], m["kv_rank"], 64, 0, 0,
+                                       700) > 0
+    assert kn.sink_attention_workspace(torch.float32, 2, 2, m["heads"], 1, m["kv_rank"] + m["rot_dim"], m["kv_rank"], 64, 0, 0,
+                                       700) == 0
+    t, u = uc.tokens(640, case.vocab, 61), uc.tokens(330, case.vocab, 62)
+    eng = case.eng
+    sa, sb = eng.new_sequence(), eng.new_sequence()
+    whole = eng.step([StepEntry(sa, t, range(600, 640)), StepEntry(sb, u, range(290, 330))]).clone()
+    eng.release(sa)
+    eng.release(sb)
+    sa, sb = eng.new_sequence(), eng.new_sequence()
+    eng.step([StepEntry(sa, t[:600], []), StepEntry(sb, u[:290], [])])
+    got = torch.cat([eng.step([StepEntry(sa, [t[600 + i]], [0]), StepEntry(sb, [u[290 + i]], [0])]).clone() for i in range(40)])
+    eng.release(sa)
+    eng.release(sb)
+    case.assert_idle()
+    got = torch.cat([got[0::2], got[1::2]])
+    want = torch.cat([case.want(t)[600:], case.want(u)[290:]])
+    noise = max(case.noise(t), case.noise(u))
+    uc.assert_close_bf16(got, want, noise)
+    uc.assert_close_bf16(got, whole.double(), noise)
+
+
 def test_a_far_key_carries_the_result(cases):
     case = cases("latent2", sharp=6.0)
     t = uc.tokens(330, case.vocab, 21)
